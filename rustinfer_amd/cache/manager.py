@@ -36,7 +36,7 @@ def pages_for(tokens: int, page_size: int) -> int:
 class KVCacheView:
     """What an attention layer gets: its layer's slice of the group's pools."""
     k: torch.Tensor          # [num_pages, num_kv_heads, page_size, head_dim]
-    v: torch.Tensor          # [num_pages, num_kv_heads, head_dim, page_size]
+    v: torch.Tensor          # [num_pages, num_kv_heads, value head_dim, page_size]
     group: int               # index into StepContext.block_tables
     page_size: int
     write: bool
@@ -66,7 +66,7 @@ class PageGroup:
             n, h, hd = len(cache_ids), need.num_kv_heads, need.head_dim
             self.k_pool = torch.zeros((n, num_pages, h, page_size, hd), device=device, dtype=dtype)
             # values are kept position-contiguous: the layout the attention kernels multiply from
-            self.v_pool = torch.zeros((n, num_pages, h, hd, page_size), device=device, dtype=dtype)
+            self.v_pool = torch.zeros((n, num_pages, h, need.value_dim, page_size), device=device, dtype=dtype)
 
     def table_row(self, rid) -> np.ndarray:
         """The request's table as an int32 array (a view of length len(table); do not write)."""
@@ -88,7 +88,7 @@ class PageGroup:
 
     def bytes_per_page(self) -> int:
         el = self.k_pool.element_size() if self.k_pool is not None else 2
-        return 2 * len(self.cache_ids) * self.need.num_kv_heads * self.page_size * self.need.head_dim * el
+        return len(self.cache_ids) * self.need.num_kv_heads * self.page_size * (self.need.head_dim + self.need.value_dim) * el
 
 
 class CacheManager:

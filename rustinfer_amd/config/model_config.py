@@ -260,3 +260,184 @@ def read_config_json(model_dir: str) -> Dict[str, Any]:
         except (OSError, json.JSONDecodeError):
             pass
     return d
+
+
+# ---------------------------------------------------------------------------
+# Tedelix: a decoder whose layers are listed one by one in config.json
+# ---------------------------------------------------------------------------
+def _obj(d: Dict[str, Any], key: str, where: str) -> Dict[str, Any]:
+    v = d.get(key)
+    if not isinstance(v, dict):
+        raise ConfigError(f"{where}: '{key}' must be an object")
+    return v
+
+
+@dataclass(frozen=True)
+class WindowAttentionSpec:
+    """Mixer ``attention``: grouped softmax attention in a sliding window, rotary angles on the
+    first ``rot_dims`` features of queries and keys, values turned by their position."""
+    heads: int
+    kv_heads: int
+    dim: int                  # size of a query / key head
+    vdim: int                 # size of a value head
+    window: int               # a query sees itself and the window - 1 positions before it
+    rot_base: float
+    rot_dims: int
+    scale: float
+    kind: str = "attention"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "WindowAttentionSpec":
+        rot, mask = _obj(m, "rot", where), _obj(m, "mask", where)
+        s = WindowAttentionSpec(
+            heads=_require(m, "heads", int, where), kv_heads=_require(m, "kv_heads", int, where),
+            dim=_require(m, "dim", int, where), vdim=_require(m, "vdim", int, where),
+            window=_require(mask, "size", int, where + ".mask"),
+            rot_base=_require(rot, "base", float, where + ".rot"), rot_dims=_require(rot, "dims", int, where + ".rot"),
+            scale=_require(m, "scale", float, where))
+        if min(s.heads, s.kv_heads, s.dim, s.vdim, s.window) <= 0 or s.heads % s.kv_heads:
+            raise ConfigError(f"{where}: heads, kv_heads, dim, vdim and mask.size must be > 0 and heads a multiple of kv_heads")
+        if s.rot_dims <= 0 or s.rot_dims % 2 or s.rot_dims > s.dim or s.vdim % 2 or not s.rot_base > 0:
+            raise ConfigError(f"{where}: rot.dims must be even and within dim, vdim even, rot.base > 0")
+        if s.dim > MAX_HEAD_DIM or s.vdim > MAX_HEAD_DIM or s.heads // s.kv_heads > 32:
+            raise ConfigError(f"{where}: heads of more than {MAX_HEAD_DIM} features or more than 32 query heads a "
+                              f"key/value head are beyond the attention kernels")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim,
+                "mask": {"size": self.window}, "rot": {"base": self.rot_base, "dims": self.rot_dims},
+                "scale": self.scale}
+
+
+@dataclass(frozen=True)
+class LightningSpec:
+    """Mixer ``lightning``: linear attention with one fixed decay for each head."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    kind: str = "lightning"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "LightningSpec":
+        decay = m.get("decay")
+        if not isinstance(decay, list):
+            raise ConfigError(f"{where}: 'decay' must be a list with one number for each head")
+        s = LightningSpec(heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where),
+                          vdim=_require(m, "vdim", int, where),
+                          decay=tuple(_typed(x, "decay", float, where) for x in decay))
+        if min(s.heads, s.dim, s.vdim) <= 0 or len(s.decay) != s.heads:
+            raise ConfigError(f"{where}: heads, dim, vdim must be > 0 and 'decay' hold {s.heads} numbers")
+        if s.dim > MAX_HEAD_DIM:
+            raise ConfigError(f"{where}: dim {s.dim} exceeds {MAX_HEAD_DIM}, the most key rows the state kernel takes")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "decay": list(self.decay)}
+
+
+@dataclass(frozen=True)
+class GeneralDeltaSpec:
+    """Mixer ``general_delta``: a generalized delta rule with a decay and a removal rate for each
+    key channel; keys, values and readers all of size ``dim``."""
+    heads: int
+    dim: int
+    # rows of the first of the two matrices behind the decay: config.json does not give it, the
+    # checkpoint's tensor does (``TedelixConfig.complete_from_checkpoint``); None: not known yet
+    decay_rank: Optional[int] = None
+    kind: str = "general_delta"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "GeneralDeltaSpec":
+        s = GeneralDeltaSpec(heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where))
+        if s.heads <= 0 or s.dim <= 0 or s.dim > MAX_HEAD_DIM:
+            raise ConfigError(f"{where}: heads must be > 0 and dim in [1, {MAX_HEAD_DIM}]")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "dim": self.dim}
+
+
+TEDELIX_MIXERS = {"attention": WindowAttentionSpec, "lightning": LightningSpec, "general_delta": GeneralDeltaSpec}
+
+
+@dataclass(frozen=True)
+class TedelixLayer:
+    mixer: Any                       # one of the specs above
+    ff: Optional[int] = None         # width of the dense feed-forward, None: the layer has none
+
+    @property
+    def type(self) -> str:
+        return self.mixer.kind
+
+
+@dataclass(frozen=True)
+class TedelixConfig(ModelConfig):
+    """``{"architecture": "Tedelix", "vocab", "width", "norm": {"eps"}, "logit_scale",
+    "logit_softcap", "layers": [{"type", "mixer": {...}, "mlp": {"kind": "dense", "ff"} | null}]}``.
+    Every layer is parallel (one norm; mixer and feed-forward read its output); the head shares
+    the embedding table; the model has no end-of-sequence token of its own."""
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    norm_eps: float = 1e-6
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
+    layers: tuple = ()
+    eos_token_ids: tuple = ()
+    architecture: str = "Tedelix"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "TedelixConfig":
+        layers_in = d.get("layers")
+        if not isinstance(layers_in, list) or not layers_in:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(layers_in):
+            w = f"{where}.layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{w}: must be an object")
+            kind = _require(entry, "type", str, w)
+            if kind not in TEDELIX_MIXERS:
+                raise ConfigError(f"{w}: unknown mixer type {kind!r} (known: {', '.join(sorted(TEDELIX_MIXERS))})")
+            mixer = TEDELIX_MIXERS[kind].from_dict(_obj(entry, "mixer", w), w + ".mixer")
+            mlp, ff = entry.get("mlp"), None
+            if mlp is not None:
+                if not isinstance(mlp, dict) or mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"{w}: 'mlp' must be null or an object of kind 'dense'")
+                ff = _require(mlp, "ff", int, w + ".mlp")
+                if ff <= 0:
+                    raise ConfigError(f"{w}.mlp: ff must be > 0")
+            layers.append(TedelixLayer(mixer, ff))
+        eos = d.get("eos_token_id")
+        eos_ids = () if eos is None else tuple(_typed(e, "eos_token_id", int, where) for e in (eos if isinstance(eos, list) else [eos]))
+        cfg = cls(vocab_size=_require(d, "vocab", int, where), hidden_size=_require(d, "width", int, where),
+                  norm_eps=_require(_obj(d, "norm", where), "eps", float, where + ".norm"),
+                  logit_scale=_typed(d.get("logit_scale", 1.0), "logit_scale", float, where),
+                  logit_softcap=_typed(d.get("logit_softcap", 0.0), "logit_softcap", float, where),
+                  layers=tuple(layers), eos_token_ids=eos_ids)
+        if cfg.vocab_size <= 0 or cfg.hidden_size <= 0 or not cfg.norm_eps > 0 or cfg.logit_softcap < 0:
+            raise ConfigError(f"{where}: vocab and width must be > 0, norm.eps > 0, logit_softcap >= 0")
+        return cfg
+
+    def complete_from_checkpoint(self, shapes: Dict[str, Any]) -> "TedelixConfig":
+        """The sizes that only a tensor's shape gives (``shapes``: checkpoint name -> shape): the
+        rank of each delta-rule layer's decay input, the rows of ``l<i>.mix.w1``."""
+        layers = []
+        for i, layer in enumerate(self.layers):
+            shape = shapes.get(f"l{i}.mix.w1")
+            if isinstance(layer.mixer, GeneralDeltaSpec) and shape is not None and len(shape) == 2:
+                layer = TedelixLayer(GeneralDeltaSpec(layer.mixer.heads, layer.mixer.dim, int(shape[0])), layer.ff)
+            layers.append(layer)
+        return TedelixConfig(**{**self.__dict__, "layers": tuple(layers)})
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {
+            "architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+            "norm": {"eps": self.norm_eps}, "logit_scale": self.logit_scale, "logit_softcap": self.logit_softcap,
+            "layers": [{"type": l.type, "mixer": l.mixer.to_dict(),
+                        "mlp": None if l.ff is None else {"kind": "dense", "ff": l.ff}} for l in self.layers]}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

@@ -56,6 +56,11 @@ def resolve_architecture(config_dict: Dict[str, Any], where: str = "config.json"
         hint = archs[0]
         if hint in _ARCHITECTURES:
             return _ARCHITECTURES[hint]
+    one = config_dict.get("architecture")          # configurations that name one architecture, as a string
+    if isinstance(one, str):
+        if one in _ARCHITECTURES:
+            return _ARCHITECTURES[one]
+        hint = hint or one
     mt = config_dict.get("model_type")
     if isinstance(mt, str):
         if mt in _MODEL_TYPE_ALIASES:
@@ -71,7 +76,19 @@ def load_model_config(model_dir: str):
     """Read ``model_dir/config.json`` -> (registry entry, typed config)."""
     d = read_config_json(model_dir)
     entry = resolve_architecture(d, where=f"{model_dir}/config.json")
-    return entry, entry.config_cls.from_dict(d, where=f"{model_dir}/config.json")
+    config = entry.config_cls.from_dict(d, where=f"{model_dir}/config.json")
+    complete = getattr(config, "complete_from_checkpoint", None)
+    if complete is not None:
+        # a design whose config.json leaves a size to the tensors' shapes: read the checkpoint's header
+        import os
+        from ..weights.safetensors_io import SafetensorsReader, WeightError
+        if any(f.endswith(".safetensors") for f in os.listdir(model_dir)):
+            try:
+                reader = SafetensorsReader(model_dir)
+                config = complete({n: tuple(reader.info(n)[1]) for n in reader.names()})
+            except WeightError:
+                pass                       # the loader will say what is wrong with the checkpoint
+    return entry, config
 
 
 _builtin_done = False
@@ -83,3 +100,4 @@ def _ensure_builtin() -> None:
         return
     _builtin_done = True
     from ..models import llama  # noqa: F401  (registers LlamaForCausalLM)
+    from ..models import tedelix  # noqa: F401  (registers Tedelix)

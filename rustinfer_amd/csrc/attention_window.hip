@@ -1,0 +1,391 @@
+// Softmax attention over the paged cache for key heads of size dk and value heads of another
+// size dv, inside a sliding window, with values that carry their position:
+//
+//   the value of position j is cached turned by j (pair m by the angle j * f_m), and the weighted
+//   sum a query at position i collects is turned back by i, so that a value enters the output
+//   turned by (j - i): a position code on the values that needs no second look at them.
+//
+// Query token t of request row b at position p, head h (key/value head g = h / (H / Hkv)):
+//   keys j in [max(0, p + 1 - window), min(kv_len_b, p + 1)),  s_j = (q . K_j) * scale,
+//   out = turn(-p) sum_j softmax(s)_j V_j.
+// Storage is 32-bit or bfloat16; scores, weights, sums and the turns are 32-bit.
+// Cache layout: keys [pages][Hkv][page][dk], values [pages][Hkv][dv][page] (positions of a
+// feature contiguous).
+//
+// rotate_kv_write: one block a token; rotates q in place over its first `rot` features (feature
+// i with i + rot/2), writes the rotated key and the turned value into the token's page.
+//
+// attn_window: a block of four waves owns up to 32 query rows: TQ = 32 / G consecutive tokens of
+// one request (G = H / Hkv query heads each) on one key/value head; a row of one token is a tile
+// of its own.  Keys go by in blocks of NK (64 where LDS allows) aligned to absolute positions, so
+// that what a query row adds up, and in which order, depends on its position alone and not on how
+// the request was cut into steps or what else the step holds.  A block of keys and values is
+// brought into LDS as 32-bit by all threads; a wave then works on four of its rows at a time
+// with one key a lane for the scores and one value feature a lane (up to four) for the sums;
+// each block of keys leaves a partial result that is merged into the row's running one.
+#include "common.h"
+#include <math.h>
+
+namespace {
+
+constexpr int AW_ROWS = 32;
+
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_kv_write_kernel(
+        T* __restrict__ q, int q_stride, const T* __restrict__ k, int k_stride, const T* __restrict__ v, int v_stride,
+        int H, int Hkv, int dk, int dv, int rot, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved,
+        const int* __restrict__ positions, const int* __restrict__ row_of_token,
+        T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ table, int max_blocks, int page, int write_kv) {
+    const int t = blockIdx.x;
+    const int b = row_of_token[t];
+    if (b < 0) return;                       // padding token
+    const int pos = positions[t];
+    const int half = rot >> 1;
+    const bool rotate = cos_t != nullptr;
+    const float* cs = rotate ? cos_t + (size_t)pos * half : nullptr;
+    const float* sn = rotate ? sin_t + (size_t)pos * half : nullptr;
+    T* qrow = q + (size_t)t * q_stride;
+    const int q_pairs = rotate ? H * half : 0;
+    for (int idx = threadIdx.x; idx < q_pairs; idx += 256) {
+        const int h = idx / half, i = idx - h * half;
+        T* qh = qrow + h * dk;
+        const float a = ld_f32(qh + i), bb = ld_f32(qh + i + half);
+        const float c = cs[i], s = sn[i];
+        st_f32(qh + i, a * c - bb * s);
+        st_f32(qh + i + half, bb * c + a * s);
+    }
+    if (!write_kv) return;
+    const int blk = table[(size_t)b * max_blocks + pos / page];
+    if (blk < 0) return;
+    const int slot = pos % page;
+    const T* krow = k + (size_t)t * k_stride;
+    for (int idx = threadIdx.x; idx < Hkv * dk; idx += 256) {
+        const int g = idx / dk, dd = idx - g * dk;
+        const T* kh = krow + g * dk;
+        float val;
+        if (rotate && dd < half) val = ld_f32(kh + dd) * cs[dd] - ld_f32(kh + dd + half) * sn[dd];
+        else if (rotate && dd < rot) val = ld_f32(kh + dd) * cs[dd - half] + ld_f32(kh + dd - half) * sn[dd - half];
+        else val = ld_f32(kh + dd);
+        st_f32(kc + (((size_t)blk * Hkv + g) * page + slot) * dk + dd, val);
+    }
+    const T* vrow = v + (size_t)t * v_stride;
+    if (vcos != nullptr) {
+        const int vh = dv >> 1;
+        const float* vcs = vcos + (size_t)pos * vh;
+        const float* vsn = vsin + (size_t)pos * vh;
+        for (int idx = threadIdx.x; idx < Hkv * vh; idx += 256) {
+            const int g = idx / vh, m = idx - g * vh;
+            const int i0 = v_interleaved ? 2 * m : m, i1 = v_interleaved ? 2 * m + 1 : m + vh;
+            const float a = ld_f32(vrow + g * dv + i0), bb = ld_f32(vrow + g * dv + i1);
+            const float c = vcs[m], s = vsn[m];
+            T* base = vc + ((size_t)blk * Hkv + g) * dv * page + slot;
+            st_f32(base + (size_t)i0 * page, a * c - bb * s);
+            st_f32(base + (size_t)i1 * page, bb * c + a * s);
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < Hkv * dv; idx += 256) {
+            const int g = idx / dv, dd = idx - g * dv;
+            vc[(((size_t)blk * Hkv + g) * dv + dd) * page + slot] = vrow[idx];
+        }
+    }
+}
+
+// One row's scores against the keys of a block, one key a lane: the block's maximum, the weights
+// relative to it and their sum.  m_b = -inf (l_b = 0) if the row sees no key of the block.
+__device__ __forceinline__ float aw_block_scores(float dot, bool mine, float scale, float& m_b, float& l_b) {
+    const float sc = mine ? dot * scale : -INFINITY;
+    m_b = wave_max(sc);
+    float pj = 0.f;
+    if (m_b > -INFINITY) pj = mine ? expf(sc - m_b) : 0.f;
+    l_b = wave_sum(pj);
+    return pj;
+}
+
+template <int NC>
+__device__ __forceinline__ void aw_merge(float& m, float& l, float (&acc)[NC], float m_b, float l_b, const float (&acc_b)[NC]) {
+    if (!(m_b > -INFINITY)) return;
+    const float M = fmaxf(m, m_b);
+    const float alpha = expf(m - M);                   // 0 while nothing has been seen (m = -inf)
+    const float beta = expf(m_b - M);
+    l = l * alpha + l_b * beta;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[c] = acc[c] * alpha + acc_b[c] * beta;
+    m = M;
+}
+
+template <typename T, int NC>    // NC: 64-wide slices of the value head a lane holds
+__global__ __launch_bounds__(256) void attn_window_kernel(
+        const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
+        const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
+        const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
+        int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window, int TQ, int NK,
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+    extern __shared__ __align__(16) float lds[];
+    const int dkp = (dk + 3) & ~3, ks_stride = dkp + 4, vs_stride = dv + 1;
+    float* Qs = lds;                                   // [AW_ROWS][dkp]
+    float* Ps = Qs + AW_ROWS * dkp;                    // [AW_ROWS][NK]
+    int* koff = reinterpret_cast<int*>(Ps + AW_ROWS * NK);      // [64] key slot in the cache, -1: none
+    float* Ks = reinterpret_cast<float*>(koff + 64);   // [NK][dkp + 4]
+    float* Vs = Ks + NK * ks_stride;                   // [NK][dv + 1]
+    float* Os = Ks;                                    // [AW_ROWS][dv], after the last block of keys
+
+    const int tile = blockIdx.x, g = blockIdx.y, G = H / Hkv;
+    int b = -1, t0 = 0, nt = 0, before = 0;
+    for (int r = 0; r < num_rows; ++r) {
+        const int lo = cu_q[r], ql = cu_q[r + 1] - lo, tiles = (ql + TQ - 1) / TQ;
+        if (tile < before + tiles) {
+            b = r;
+            t0 = lo + (tile - before) * TQ;
+            nt = min(TQ, lo + ql - t0);
+            break;
+        }
+        before += tiles;
+    }
+    if (b < 0) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int R = nt * G;                              // rows in use: row r = token r / G, head g G + r % G
+    const int p0 = q_start[b] + (t0 - cu_q[b]);        // position of the tile's first token
+    const int kv_len = kv_lens[b];
+    const int last_visible = min(kv_len, p0 + nt);
+    const int first_key = window > 0 ? max(0, p0 + 1 - window) : 0;
+
+    for (int e = tid; e < AW_ROWS * dkp; e += 256) {
+        const int r = e / dkp, dd = e - r * dkp;
+        Qs[e] = (r < R && dd < dk) ? ld_f32(q + (size_t)(t0 + r / G) * q_stride + (g * G + r % G) * dk + dd) : 0.f;
+    }
+    const int batches = (R + 15) / 16;                 // the same for all waves: they share the barriers
+    float m[8], l[8], acc[8][NC];
+    int row_lo[8], row_hi[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        m[i] = -INFINITY;
+        l[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[i][c] = 0.f;
+        const int r = wave + 4 * i, p = p0 + r / G;
+        row_hi[i] = r < R ? min(kv_len, p + 1) : 0;
+        row_lo[i] = window > 0 ? max(0, p + 1 - window) : 0;
+    }
+
+    for (int kb = first_key / NK; kb * NK < last_visible; ++kb) {
+        const int j_base = kb * NK;
+        __syncthreads();                               // the last block of keys has been used (first pass: Qs is written)
+        if (tid < NK) {
+            const int j = j_base + tid;
+            int off = -1;
+            if (j < last_visible && j >= first_key) {
+                const int pid = table[(size_t)b * max_blocks + j / page];
+                if (pid >= 0) off = (pid * Hkv + g) * page + j % page;      // -1: a page the window has given back
+            }
+            koff[tid] = off;
+        }
+        __syncthreads();
+        for (int e = tid; e < NK * dkp; e += 256) {
+            const int jj = e / dkp, dd = e - jj * dkp, off = koff[jj];
+            Ks[jj * ks_stride + dd] = (off >= 0 && dd < dk) ? ld_f32(kc + (size_t)off * dk + dd) : 0.f;
+        }
+        {
+            const int jj = tid % NK, off = koff[jj];
+            const size_t vbase = off >= 0 ? (size_t)(off / page) * page * dv + off % page : 0;
+            for (int d = tid / NK; d < dv; d += 256 / NK)
+                Vs[jj * vs_stride + d] = off >= 0 ? ld_f32(vc + vbase + (size_t)d * page) : 0.f;
+        }
+        __syncthreads();
+        float m_b[8], l_b[8], acc_b[8][NC];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            m_b[i] = -INFINITY;
+            l_b[i] = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) acc_b[i][c] = 0.f;
+        }
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+            if (bi >= batches) break;
+            float s[4] = {0.f, 0.f, 0.f, 0.f};
+            const float* kr = Ks + (lane < NK ? lane : 0) * ks_stride;
+#pragma unroll 2
+            for (int dd = 0; dd < dkp; dd += 4) {
+                const float4 k4 = *reinterpret_cast<const float4*>(kr + dd);
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb) {
+                    const float4 q4 = *reinterpret_cast<const float4*>(Qs + (wave + 4 * (4 * bi + rb)) * dkp + dd);
+                    s[rb] = fmaf(q4.x, k4.x, s[rb]);
+                    s[rb] = fmaf(q4.y, k4.y, s[rb]);
+                    s[rb] = fmaf(q4.z, k4.z, s[rb]);
+                    s[rb] = fmaf(q4.w, k4.w, s[rb]);
+                }
+            }
+            const int j = j_base + lane;
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const int i = 4 * bi + rb;
+                const bool mine = lane < NK && j >= row_lo[i] && j < row_hi[i];
+                const float pj = aw_block_scores(s[rb], mine, scale, m_b[i], l_b[i]);
+                if (lane < NK) Ps[(wave + 4 * i) * NK + lane] = pj;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+            if (bi >= batches) break;
+#pragma unroll 1
+            for (int jj = 0; jj < NK; jj += 4) {
+                float4 p4[4];
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb)
+                    p4[rb] = *reinterpret_cast<const float4*>(Ps + (wave + 4 * (4 * bi + rb)) * NK + jj);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) {
+                        const int d = lane + 64 * c;
+                        const float v = d < dv ? Vs[(jj + u) * vs_stride + d] : 0.f;
+#pragma unroll
+                        for (int rb = 0; rb < 4; ++rb) {
+                            const float pv = u == 0 ? p4[rb].x : u == 1 ? p4[rb].y : u == 2 ? p4[rb].z : p4[rb].w;
+                            acc_b[4 * bi + rb][c] = fmaf(pv, v, acc_b[4 * bi + rb][c]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) aw_merge<NC>(m[i], l[i], acc[i], m_b[i], l_b[i], acc_b[i]);
+    }
+    if (vcos == nullptr) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = wave + 4 * i;
+            if (r >= R) continue;
+            T* o = out + (size_t)(t0 + r / G) * out_stride + (g * G + r % G) * dv;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const int d = lane + 64 * c;
+                if (d < dv) st_f32(o + d, l[i] > 0.f ? acc[i][c] / l[i] : 0.f);
+            }
+        }
+        return;
+    }
+    // the sums are turned back by the query's position: through LDS, since a pair's two
+    // features lie in different lanes
+    __syncthreads();                                   // the last keys and values have been used
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = wave + 4 * i;
+        if (r >= R) continue;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int d = lane + 64 * c;
+            if (d < dv) Os[r * dv + d] = l[i] > 0.f ? acc[i][c] / l[i] : 0.f;
+        }
+    }
+    __syncthreads();
+    const int vh = dv >> 1;
+    for (int r = wave; r < R; r += 4) {
+        const int p = p0 + r / G;
+        T* o = out + (size_t)(t0 + r / G) * out_stride + (g * G + r % G) * dv;
+        for (int mm = lane; mm < vh; mm += 64) {
+            const int i0 = v_interleaved ? 2 * mm : mm, i1 = v_interleaved ? 2 * mm + 1 : mm + vh;
+            const float a = Os[r * dv + i0], bb = Os[r * dv + i1];
+            const float c = vcos[(size_t)p * vh + mm], s = vsin[(size_t)p * vh + mm];
+            st_f32(o + i0, a * c + bb * s);
+            st_f32(o + i1, bb * c - a * s);
+        }
+    }
+}
+
+size_t aw_lds_bytes(int dk, int dv, int NK) {
+    const int dkp = (dk + 3) & ~3;
+    const size_t kv = (size_t)NK * (dkp + 4) + (size_t)NK * (dv + 1);
+    const size_t os = (size_t)AW_ROWS * dv;
+    return sizeof(float) * ((size_t)AW_ROWS * dkp + (size_t)AW_ROWS * NK + 64 + (kv > os ? kv : os));
+}
+
+constexpr size_t AW_LDS_MOST = 150 * 1024;
+
+}  // namespace
+
+extern "C" int ri_attention_window_supported(int H, int Hkv, int dk, int dv) {
+    return H > 0 && Hkv > 0 && H % Hkv == 0 && H / Hkv <= AW_ROWS && dk > 0 && dk <= 256 && dv > 0 && dv <= 256
+        && aw_lds_bytes(dk, dv, 16) <= AW_LDS_MOST;
+}
+
+extern "C" int ri_rotate_kv_write(
+        void* q, int q_stride, const void* k, int k_stride, const void* v, int v_stride, int dtype, int T,
+        int H, int Hkv, int dk, int dv, int rot, const float* cos_t, const float* sin_t, int table_rows,
+        const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
+        const int* positions, const int* row_of_token, void* kc, void* vc, int num_pages,
+        const int* table, int max_blocks, int page, int write_kv, hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && H > 0 && Hkv > 0 && dk > 0 && dv > 0 && page > 0, "ri_rotate_kv_write: bad sizes");
+    RI_REQUIRE(q_stride >= H * dk, "ri_rotate_kv_write: query row stride %d too small", q_stride);
+    if (cos_t) RI_REQUIRE(rot > 0 && rot % 2 == 0 && rot <= dk && sin_t && table_rows > 0, "ri_rotate_kv_write: rot %d must be even and within the key size %d", rot, dk);
+    if (vcos) RI_REQUIRE(dv % 2 == 0 && vsin && v_table_rows > 0, "ri_rotate_kv_write: a turned value needs an even size, got %d", dv);
+    if (write_kv) RI_REQUIRE(k && v && kc && vc && table && max_blocks > 0 && num_pages > 0 && k_stride >= Hkv * dk && v_stride >= Hkv * dv,
+                             "ri_rotate_kv_write: no keys, values or cache given, or their row strides too small");
+    if (T == 0) return 0;
+    RI_REQUIRE(q && positions && row_of_token, "ri_rotate_kv_write: null pointer");
+    if (dtype == RI_F32)
+        rotate_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, H, Hkv, dk, dv, rot, cos_t, sin_t, vcos, vsin, v_interleaved, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv);
+    else if (dtype == RI_BF16)
+        rotate_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, Hkv, dk, dv, rot, cos_t, sin_t, vcos, vsin, v_interleaved, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv);
+    else
+        return ri_fail("ri_rotate_kv_write: unknown dtype %d", dtype);
+    RI_LAUNCHED("ri_rotate_kv_write");
+    return 0;
+}
+
+namespace {
+template <typename T>
+int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
+              const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
+              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, hipStream_t stream) {
+    const int G = H / Hkv, TQ = AW_ROWS / G;
+    int NK = 64;
+    while (NK > 16 && aw_lds_bytes(dk, dv, NK) > AW_LDS_MOST) NK >>= 1;
+    const size_t lds = aw_lds_bytes(dk, dv, NK);
+    const int NC = (dv + 63) / 64;
+    auto kernel = NC == 1 ? attn_window_kernel<T, 1> : NC == 2 ? attn_window_kernel<T, 2> : NC == 3 ? attn_window_kernel<T, 3> : attn_window_kernel<T, 4>;
+    if (lds > 64 * 1024) {
+        // more LDS than a kernel gets unasked: requested once for each form of the kernel
+        static bool asked[5] = {};
+        if (!asked[NC]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)AW_LDS_MOST);
+            RI_REQUIRE(e == hipSuccess, "ri_attention_window: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+            asked[NC] = true;
+        }
+    }
+    const int tiles = (Tn + TQ - 1) / TQ + num_rows;   // at most: every request may end in a short tile
+    kernel<<<dim3(tiles, Hkv), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens,
+                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved);
+    return 0;
+}
+}  // namespace
+
+// Attention of the step's tokens (rotated queries in q) over the cache; out [T][>= H dv].
+// vcos / vsin [positions][dv / 2]: the sums are turned back by the query's position (null: not).
+extern "C" int ri_attention_window(
+        const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kc, const void* vc,
+        int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
+        const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
+        float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
+        hipStream_t stream) {
+    RI_REQUIRE(ri_attention_window_supported(H, Hkv, dk, dv), "ri_attention_window: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
+    RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window: bad sizes");
+    RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window: row strides too small");
+    if (vcos) RI_REQUIRE(vsin && dv % 2 == 0 && v_table_rows > 0, "ri_attention_window: a turned value needs an even size and both tables");
+    if (T == 0 || num_rows == 0) return 0;
+    RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_window: null pointer");
+    RI_REQUIRE(Hkv <= 65535, "ri_attention_window: too many key/value heads for the grid");
+    int rc;
+    if (dtype == RI_F32)
+        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+    else if (dtype == RI_BF16)
+        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+    else
+        return ri_fail("ri_attention_window: unknown dtype %d", dtype);
+    if (rc) return rc;
+    RI_LAUNCHED("ri_attention_window");
+    return 0;
+}

@@ -448,3 +448,55 @@ extern "C" int ri_swiglu(const void* gate_up, void* out, int act_dtype, int T, i
     RI_LAUNCHED("ri_swiglu");
     return 0;
 }
+
+// ---------------------------------------------------------------------------
+// out[t, i] = f(in[t, i]) over n columns of rows with strides of their own (columns of a wider
+// buffer; in place where out == in).  f: 0 = relu(z)^2, 1 = tanh(z); 32-bit arithmetic.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void unary_kernel(const T* __restrict__ in, int in_stride, T* __restrict__ out,
+                                                    int out_stride, int n, int op) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float z = ld_f32(in + (size_t)t * in_stride + i);
+    float y;
+    if (op == 0) { const float r = fmaxf(z, 0.f); y = r * r; }
+    else y = tanhf(z);
+    st_f32(out + (size_t)t * out_stride + i, y);
+}
+
+extern "C" int ri_unary(const void* in, int in_stride, void* out, int out_stride, int dtype, int T, int n, int op,
+                        hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && n > 0 && in_stride >= n && out_stride >= n, "ri_unary: bad sizes T=%d n=%d", T, n);
+    RI_REQUIRE(op == 0 || op == 1, "ri_unary: unknown function %d", op);
+    if (T == 0) return 0;
+    RI_REQUIRE(in && out, "ri_unary: null pointer");
+    RI_REQUIRE(T <= 65535, "ri_unary: too many rows for the grid");
+    dim3 grid((n + 255) / 256, T);
+    if (dtype == RI_F32) unary_kernel<float><<<grid, 256, 0, stream>>>((const float*)in, in_stride, (float*)out, out_stride, n, op);
+    else if (dtype == RI_BF16) unary_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)in, in_stride, (bf16_t*)out, out_stride, n, op);
+    else return ri_fail("ri_unary: unknown dtype %d", dtype);
+    RI_LAUNCHED("ri_unary");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// logits <- cap * tanh(logits * scale / cap) in place (cap <= 0: logits * scale only).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void scale_softcap_kernel(float* __restrict__ x, size_t n, float scale, float cap) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float z = x[i] * scale;
+    x[i] = cap > 0.f ? cap * tanhf(z / cap) : z;
+}
+
+extern "C" int ri_scale_softcap(float* x, int rows, int cols, float scale, float cap, hipStream_t stream) {
+    RI_REQUIRE(rows >= 0 && cols > 0, "ri_scale_softcap: bad sizes");
+    if (rows == 0) return 0;
+    RI_REQUIRE(x, "ri_scale_softcap: null pointer");
+    const size_t n = (size_t)rows * cols;
+    scale_softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, n, scale, cap);
+    RI_LAUNCHED("ri_scale_softcap");
+    return 0;
+}

@@ -46,7 +46,7 @@ def pages_that_fit(needs, page_size: int, element_size: int, free_bytes: int, me
     per_page = state = 0
     for need in needs.values():
         if isinstance(need, PagedKVNeed):
-            per_page += 2 * need.num_kv_heads * need.head_dim * page_size * element_size
+            per_page += need.num_kv_heads * (need.head_dim + need.value_dim) * page_size * element_size
         elif isinstance(need, StateNeed):
             n = 1
             for d in need.shape:
@@ -90,7 +90,7 @@ def second_copy_budget(model, rt: Runtime, page_size: int, num_pages: int, max_r
     # what the allocator holds and does not use is free to it as well
     free += max(0, torch.cuda.memory_reserved(rt.device) - torch.cuda.memory_allocated(rt.device))
     if num_pages > 0:
-        cache = sum(2 * need.num_kv_heads * need.head_dim * page_size * el * (num_pages + 1)
+        cache = sum(need.num_kv_heads * (need.head_dim + need.value_dim) * page_size * el * (num_pages + 1)
                     for need in model.cache_needs().values() if isinstance(need, PagedKVNeed))
     else:
         cache = int(reserve * total)
@@ -131,7 +131,7 @@ def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: i
     engine = Engine(model, rt, page_size=page_size, num_pages=bootstrap, max_requests=max_requests,
                     max_model_len=max_model_len, max_batch_tokens=max_batch_tokens)
     engine.profile_forward()
-    held = sum(g.k_pool.numel() * g.k_pool.element_size() * 2 for g in engine.cache.groups) + engine.cache.state_bytes()
+    held = sum((g.k_pool.numel() + g.v_pool.numel()) * g.k_pool.element_size() for g in engine.cache.groups) + engine.cache.state_bytes()
     # the state tensors are part of what auto_num_pages subtracts; the bootstrap's own go back with its pool
     num_pages = auto_num_pages(model, rt, page_size, mem_fraction, max_requests, max_model_len, held_bytes=held)
     engine.resize_pool(num_pages)

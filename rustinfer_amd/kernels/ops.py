@@ -648,7 +648,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
 
 
 def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
-                 w_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 w_tiled: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``x @ w^T`` as a residual delta for ``add_rmsnorm``: ``[M, N]`` in the dtype of ``x``, or,
     for few bfloat16 rows and few output columns, a float32 stack ``[P, M, N]`` of partial sums
     over slices of K (so that the product still fills the chip) which the norm adds up."""
@@ -679,7 +679,7 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
                                            _ptr(stack), N, M, N, K, F32, 0, parts, ctypes.c_longlong(M * N),
                                            int(tiled), ctypes.c_void_p(0), 0, ctypes.c_float(0.0), _stream()))
             return stack
-    out = workspace.get(name, M, N, x.dtype)
+    out = workspace.get(name, M, N, out_dtype or x.dtype)     # out_dtype: 32-bit sums of a bfloat16 product left unrounded
     linear(x, w, out, w_tiled)
     return out
 
@@ -807,3 +807,192 @@ def measure_peaks(device="cuda:0", read_bytes: int = 4 << 30, reps: int = 5):
             e1.synchronize()
             out[name] = round(work.value * reps / (e0.elapsed_time(e1) * 1e-3) / unit, 1)
     return out
+
+
+# ---------------------------------------------------------------------------
+# elementwise functions on columns of a wider buffer, the output head's soft cap
+# ---------------------------------------------------------------------------
+UNARY = {"relu2": 0, "tanh": 1}
+
+
+def unary(name: str, x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = f(x)`` for ``f`` in ``UNARY`` (the square of relu, tanh), 32-bit arithmetic; ``x`` and
+    ``out`` are ``[T, n]`` with unit column stride and any row stride (``out`` may be ``x``)."""
+    _dev(x, out)
+    _rows2d(x, "x")
+    _rows2d(out, "out")
+    if name not in UNARY or x.shape != out.shape or x.dtype != out.dtype:
+        raise KernelError(f"unary: unknown function {name!r}, or shapes / dtypes differ")
+    T, n = x.shape
+    _check(_lib().ri_unary(_ptr(x), x.stride(0), _ptr(out), out.stride(0), _dt(x), T, n, UNARY[name], _stream()))
+
+
+def scale_softcap(logits: torch.Tensor, scale: float, cap: float) -> None:
+    """``logits <- cap * tanh(logits * scale / cap)`` in place (``cap <= 0``: the scale alone)."""
+    _dev(logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+        raise KernelError("scale_softcap: logits must be contiguous float32 [rows, vocab]")
+    _check(_lib().ri_scale_softcap(_ptr(logits), logits.shape[0], logits.shape[1], ctypes.c_float(scale),
+                                   ctypes.c_float(cap), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# attention with key and value heads of different sizes, a window and turned values
+# ---------------------------------------------------------------------------
+def _rot_tables(tables, size: int, who: str):
+    """(cos, sin, rows) pointers of a rotation's tables ``[positions, size / 2]``, or nulls."""
+    if tables is None:
+        return ctypes.c_void_p(0), ctypes.c_void_p(0), 0
+    cos, sin = tables[0], tables[1]
+    _dev(cos, sin)
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2 \
+            or cos.shape[1] * 2 != size or not cos.is_contiguous() or not sin.is_contiguous():
+        raise KernelError(f"{who}: cos/sin must be contiguous float32 [positions, {size // 2}]")
+    return _ptr(cos), _ptr(sin), cos.shape[0]
+
+
+def _check_cache_kv(k_cache, v_cache, Hkv, dk, dv, page, act_dtype, name):
+    if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (Hkv, page, dk) or v_cache.dim() != 4 \
+            or tuple(v_cache.shape) != (k_cache.shape[0], Hkv, dv, page):
+        raise KernelError(f"{name}: caches must be k [pages, {Hkv}, {page}, {dk}] and v [pages, {Hkv}, {dv}, {page}], "
+                          f"got {tuple(k_cache.shape)} and {tuple(v_cache.shape)}")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise KernelError(f"{name}: cache must be contiguous")
+    if k_cache.dtype != act_dtype or v_cache.dtype != act_dtype:
+        raise KernelError(f"{name}: cache dtype {k_cache.dtype} differs from the activations' {act_dtype}")
+
+
+def rotate_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], H: int, Hkv: int,
+                    dk: int, dv: int, rotary, value_rotary, positions: torch.Tensor, row_of_token: torch.Tensor,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, page: int,
+                    write_kv: bool = True, interleaved_values: bool = False) -> None:
+    """Rotate ``q [T, H dk]`` in place (``rotary = (cos, sin, rot_dim)``: the first ``rot_dim``
+    features of a head, feature i with i + rot_dim/2) and write this step's keys (rotated the same
+    way) and values into their pages.  ``value_rotary = (cos, sin)`` ``[positions, dv/2]``: a value
+    is cached turned by its position over all its features, pair m = (m, m + dv/2), or
+    (2m, 2m + 1) with ``interleaved_values``.  q, k, v may be columns of one wider buffer."""
+    _dev(q, k, v, positions, row_of_token, k_cache, v_cache, block_table)
+    _rows2d(q, "q")
+    T = q.shape[0]
+    if q.shape[1] != H * dk:
+        raise KernelError(f"rotate_kv_write: q must be [T, {H * dk}]")
+    _i32(positions, "positions", T)
+    _i32(row_of_token, "row_of_token", T)
+    rot = 0
+    cos = sin = ctypes.c_void_p(0)
+    rows = 0
+    if rotary is not None:
+        rot = int(rotary[2])
+        cos, sin, rows = _rot_tables(rotary, rot, "rotate_kv_write")
+    vcos, vsin, vrows = _rot_tables(value_rotary, dv, "rotate_kv_write (values)")
+    if write_kv:
+        _rows2d(k, "k")
+        _rows2d(v, "v")
+        if tuple(k.shape) != (T, Hkv * dk) or tuple(v.shape) != (T, Hkv * dv) or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise KernelError(f"rotate_kv_write: k must be [T, {Hkv * dk}] and v [T, {Hkv * dv}] of {q.dtype}")
+        _check_cache_kv(k_cache, v_cache, Hkv, dk, dv, page, q.dtype, "rotate_kv_write")
+        _i32(block_table, "block_table")
+        if block_table.dim() != 2:
+            raise KernelError("rotate_kv_write: block_table must be [rows, max_blocks]")
+    _check(_lib().ri_rotate_kv_write(
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0) if k is not None else 0, _ptr(v), v.stride(0) if v is not None else 0,
+        _dt(q), T, H, Hkv, dk, dv, rot, cos, sin, rows, vcos, vsin, vrows, int(bool(interleaved_values)),
+        _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache),
+        k_cache.shape[0] if k_cache is not None else 0, _ptr(block_table),
+        block_table.shape[1] if block_table is not None and block_table.dim() == 2 else 0, page,
+        int(bool(write_kv)), _stream()))
+
+
+def window_attention_supported(H: int, Hkv: int, dk: int, dv: int) -> bool:
+    return bool(_lib().ri_attention_window_supported(H, Hkv, dk, dv))
+
+
+def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: int, dv: int,
+                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, page: int,
+                     ctx, scale: float, window: int = 0, value_rotary=None,
+                     interleaved_values: bool = False) -> None:
+    """Attention of the step's tokens (rotated queries ``q [T, H dk]``) over the cache into
+    ``out [T, H dv]``: keys of size ``dk``, values of size ``dv``, the last ``window`` positions
+    (0: all).  ``value_rotary``: the cached values are turned by their positions, and each sum is
+    turned back by its query's."""
+    _dev(q, out, k_cache, v_cache, block_table)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    T = q.shape[0]
+    if q.shape[1] != H * dk or tuple(out.shape) != (T, H * dv) or out.dtype != q.dtype:
+        raise KernelError(f"window_attention: q must be [T, {H * dk}] and out [T, {H * dv}] of one dtype")
+    _check_cache_kv(k_cache, v_cache, Hkv, dk, dv, page, q.dtype, "window_attention")
+    _i32(block_table, "block_table")
+    if block_table.dim() != 2 or block_table.shape[0] < ctx.num_rows:
+        raise KernelError("window_attention: block_table must be [rows, max_blocks]")
+    _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+    _i32(ctx.q_start, "q_start", ctx.num_rows)
+    _i32(ctx.kv_lens, "kv_lens", ctx.num_rows)
+    vcos, vsin, vrows = _rot_tables(value_rotary, dv, "window_attention (values)")
+    _check(_lib().ri_attention_window(
+        _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
+        H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
+        ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# mixers with a matrix of state for each head
+# ---------------------------------------------------------------------------
+def linear_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, out: torch.Tensor, ctx,
+                H: int, dk: int, dv: int, decay: Optional[torch.Tensor] = None, silu_in: bool = False,
+                wl: Optional[torch.Tensor] = None, al: Optional[torch.Tensor] = None,
+                w0: Optional[torch.Tensor] = None, ab: Optional[torch.Tensor] = None,
+                unit_eps: float = 1e-6, decay_c: float = 1.0) -> None:
+    """Walk each request's tokens of the step through its state ``state[slot] [H, dk, dv]`` (32-bit):
+    ``S <- diag(w) S - (a u)(u^T S) + k v^T``, ``out_t = S^T r`` (32-bit ``[T, H dv]``).
+    With ``decay [H]``: ``w`` is the head's constant, no second term, and r, k, v pass through silu if
+    ``silu_in``.  With ``wl, al [T, H dk]`` and 32-bit ``w0, ab [H dk]``: ``u = k / sqrt(|k|^2 + unit_eps)``,
+    ``w = exp(-decay_c sigmoid(wl + w0))``, ``a = sigmoid(al + ab)``.  A request's first tokens
+    (``q_start == 0``) start from zeros."""
+    _dev(r, k, v, state, out, decay, wl, al, w0, ab)
+    for t, name in ((r, "r"), (k, "k"), (v, "v"), (out, "out")):
+        _rows2d(t, name)
+    T = r.shape[0]
+    delta = decay is None
+    if tuple(r.shape) != (T, H * dk) or tuple(k.shape) != (T, H * dk) or tuple(v.shape) != (T, H * dv) \
+            or tuple(out.shape) != (T, H * dv) or out.dtype != torch.float32 or k.dtype != r.dtype or v.dtype != r.dtype:
+        raise KernelError("linear_scan: r, k [T, H dk], v [T, H dv] of one dtype and 32-bit out [T, H dv] expected")
+    if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (H, dk, dv) or not state.is_contiguous():
+        raise KernelError(f"linear_scan: state must be contiguous float32 [slots, {H}, {dk}, {dv}]")
+    if delta:
+        for t, name in ((wl, "wl"), (al, "al")):
+            if t is None or tuple(t.shape) != (T, H * dk) or t.dtype != r.dtype or t.stride(1) != 1:
+                raise KernelError(f"linear_scan: {name} must be [T, {H * dk}] of {r.dtype}")
+        for t, name in ((w0, "w0"), (ab, "ab")):
+            if t is None or t.dtype != torch.float32 or t.numel() != H * dk or not t.is_contiguous():
+                raise KernelError(f"linear_scan: {name} must be contiguous float32 with {H * dk} entries")
+    elif decay.dtype != torch.float32 or decay.numel() != H or not decay.is_contiguous():
+        raise KernelError(f"linear_scan: decay must be contiguous float32 with {H} entries")
+    _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+    _i32(ctx.q_start, "q_start", ctx.num_rows)
+    _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+    _check(_lib().ri_linear_scan(
+        _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
+        _ptr(wl), wl.stride(0) if wl is not None else 0, _ptr(al), al.stride(0) if al is not None else 0, _dt(r),
+        _ptr(w0), _ptr(ab), _ptr(decay), int(delta), int(bool(silu_in)), ctypes.c_float(unit_eps),
+        ctypes.c_float(decay_c), _ptr(state), state.shape[0], _ptr(out), out.stride(0),
+        _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.state_slots), ctx.num_rows, T, H, dk, dv, _stream()))
+
+
+def gated_group_norm(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor,
+                     group: int, eps: float) -> None:
+    """``out = o / sqrt(mean over each group of `group` features (o^2) + eps) * weight * sigmoid(gate)``;
+    ``o`` 32-bit ``[T, n]``, ``gate`` and ``out`` activations (columns of wider buffers allowed)."""
+    _dev(o, weight, gate, out)
+    _rows2d(o, "o")
+    _rows2d(out, "out")
+    T, n = o.shape
+    if o.dtype != torch.float32 or tuple(out.shape) != (T, n) or weight.numel() != n or not weight.is_contiguous():
+        raise KernelError("gated_group_norm: 32-bit o [T, n], out [T, n] and n weights expected")
+    if gate is not None:
+        _rows2d(gate, "gate")
+        if tuple(gate.shape) != (T, n) or gate.dtype != out.dtype:
+            raise KernelError("gated_group_norm: gate must be [T, n] in the dtype of out")
+    _check(_lib().ri_gated_group_norm(_ptr(o), o.stride(0), T, n, int(group), _ptr(weight), _dt(weight), _ptr(gate),
+                                      gate.stride(0) if gate is not None else 0, _ptr(out), out.stride(0), _dt(out),
+                                      ctypes.c_float(eps), _stream()))

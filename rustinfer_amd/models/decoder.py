@@ -15,7 +15,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import ParamSpec, Part, PositionEncoding, Runtime, narrow_tensors
+from ..parts.base import ParamSpec, Part, PositionEncoding, Runtime, join_name, narrow_tensors
 from ..parts.block import Hidden
 from ..parts.embed import Embedding, LMHead
 
@@ -66,7 +66,7 @@ class DecoderModel(Part):
         specs: Dict[str, ParamSpec] = {}
         for prefix, part in self._children():
             for name, spec in part.param_specs().items():
-                specs[f"{prefix}.{name}"] = spec
+                specs[join_name(prefix, name)] = spec
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:

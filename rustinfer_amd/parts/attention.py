@@ -16,7 +16,8 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import DeferredNorm, Mixer, PagedKVNeed, ParamSpec, PositionEncoding, Runtime, split_normed
+from .base import (DeferredNorm, Mixer, PagedKVNeed, ParamSpec, PositionEncoding, ProjectedPart, Runtime,
+                   split_normed)
 from .linear import Linear
 
 
@@ -150,3 +151,61 @@ class PagedAttention(Mixer):
                             cache.k, cache.v, table, cache.page_size, ctx, self.scale,
                             self.window or 0)
         return attn
+
+
+class WindowAttention(ProjectedPart, Mixer):
+    """Grouped softmax attention over the last ``window`` positions with key heads of size
+    ``head_dim`` and value heads of size ``v_head_dim``.  ``pos_enc`` rotates the first
+    ``pos_enc.rot_dim`` features of queries and keys; ``value_pos_enc`` (a rotation over all of
+    ``v_head_dim``) is applied to every value before it is cached, by the value's position, and
+    undone on each head's sum by the query's position, so that a value enters the output turned by
+    the distance between the two.  Scores are ``(q . k) * scale``; the softmax is over the visible
+    keys only.  Tensor names: ``q, k, v, o`` unless given."""
+
+    is_mixer = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
+                 scale: float, window: Optional[int] = None, pos_enc: Optional[PositionEncoding] = None,
+                 value_pos_enc: Optional[PositionEncoding] = None, interleaved_values: bool = False,
+                 names: Optional[Dict[str, str]] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.num_kv_heads = int(num_heads), int(num_kv_heads)
+        self.head_dim, self.v_head_dim = int(head_dim), int(v_head_dim)
+        self.scale = float(scale)
+        self.window = int(window) if window else None
+        self.pos_enc, self.value_pos_enc = pos_enc, value_pos_enc
+        self.interleaved_values = bool(interleaved_values)
+        self.names = {"q": "q", "k": "k", "v": "v", "o": "o"}
+        if names:
+            self.names.update(names)
+
+    def in_projections(self):
+        n = self.names
+        return [(n["q"], self.num_heads * self.head_dim), (n["k"], self.num_kv_heads * self.head_dim),
+                (n["v"], self.num_kv_heads * self.v_head_dim)]
+
+    def out_projection(self):
+        return (self.names["o"], self.num_heads * self.v_head_dim)
+
+    def cache_need(self):
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window, self.v_head_dim)
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        if not rt.ops.window_attention_supported(self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim):
+            raise ValueError(f"attention with {self.num_heads}/{self.num_kv_heads} heads of {self.head_dim} and "
+                             f"{self.v_head_dim} features is beyond the window attention kernel")
+
+    def core(self, ctx, proj, act, cache) -> None:
+        ops, n = self.rt.ops, self.names
+        q, k, v = proj[n["q"]], proj[n["k"]], proj[n["v"]]
+        table = ctx.block_tables[cache.group]
+        rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
+        vrot = self.value_pos_enc.rotary()[:2] if self.value_pos_enc is not None else None
+        ops.rotate_kv_write(q, k, v, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, rotary, vrot,
+                            ctx.positions, ctx.row_of_token, cache.k, cache.v, table, cache.page_size,
+                            write_kv=cache.write, interleaved_values=self.interleaved_values)
+        ops.window_attention(q, act, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, cache.k, cache.v,
+                             table, cache.page_size, ctx, self.scale, self.window or 0, vrot, self.interleaved_values)

@@ -44,7 +44,7 @@ between two sub-layers needs no kernel of its own when a step has few tokens:
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Optional, Tuple
+from typing import Any, Callable, Dict, List, Optional, Tuple
 
 import torch
 
@@ -65,10 +65,16 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class PagedKVNeed:
-    """Keys and values of every position (or of the last ``window`` positions)."""
+    """Keys and values of every position (or of the last ``window`` positions).  ``v_head_dim``:
+    the size of a value head where it differs from a key head's."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
@@ -99,6 +105,14 @@ def split_normed(normed):
     return normed, None
 
 
+def join_name(prefix: str, name: str) -> str:
+    """A part's tensor under its parent's prefix; a part whose one tensor carries the part's own
+    name (no suffix) calls it ``""``."""
+    if not prefix:
+        return name
+    return f"{prefix}.{name}" if name else prefix
+
+
 class LazyTensors:
     """name -> tensor for ``load``: a tensor is made when it is asked for and not kept, so that a
     model can be filled part by part without all of its tensors existing at once beside it."""
@@ -107,16 +121,19 @@ class LazyTensors:
         self._names, self._make, self._prefix = names, make, prefix
 
     def __getitem__(self, name: str) -> torch.Tensor:
-        full = self._prefix + name
+        full = join_name(self._prefix, name)
         if full not in self._names:
             raise KeyError(name)
         return self._make(full)
 
     def __contains__(self, name) -> bool:
-        return self._prefix + str(name) in self._names
+        return join_name(self._prefix, str(name)) in self._names
 
     def keys(self):
-        return [n[len(self._prefix):] for n in self._names if n.startswith(self._prefix)]
+        if not self._prefix:
+            return list(self._names)
+        dot = self._prefix + "."
+        return [n[len(dot):] for n in self._names if n.startswith(dot)] + ([""] if self._prefix in self._names else [])
 
     def __iter__(self):
         return iter(self.keys())
@@ -128,14 +145,17 @@ class LazyTensors:
         return ((n, self[n]) for n in self.keys())
 
     def narrow(self, prefix: str) -> "LazyTensors":
-        return LazyTensors(self._names, self._make, self._prefix + prefix + ".")
+        return LazyTensors(self._names, self._make, join_name(self._prefix, prefix))
 
 
 def narrow_tensors(tensors, prefix: str):
     """The tensors whose names begin with ``prefix.``, under the rest of their names."""
     if hasattr(tensors, "narrow"):
         return tensors.narrow(prefix)
-    return {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
+    sub = {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
+    if prefix in tensors:
+        sub[""] = tensors[prefix]          # the part's one tensor carries the part's own name
+    return sub
 
 
 @dataclass
@@ -240,3 +260,147 @@ def stored_to(t: torch.Tensor, rt: Runtime, keep_fp32: bool = False) -> torch.Te
     if keep_fp32 and t.dtype == torch.float32:
         return t.to(device=rt.device).contiguous()
     return t.to(device=rt.device, dtype=rt.dtype).contiguous()
+
+
+# ---------------------------------------------------------------------------
+# Sub-layers of the shape  out = W_out f(W_in n)
+# ---------------------------------------------------------------------------
+class ProjectedPart(Part):
+    """A mixer or feed-forward whose first step is a set of projections of its input and whose
+    last is one projection back to the model's width, with anything in between (``core``).
+
+    A part that says so lets whoever owns it stack the projections of several parts that read the
+    same input into one product, and their output projections into one product over the
+    concatenated activations (a block whose mixer and feed-forward read the same norm); used on its
+    own it behaves as any other part (``param_specs`` / ``load`` / ``forward``).
+
+    ``in_projections()``  [(tensor name, rows)]: weights ``[rows, hidden]`` applied to the input.
+    ``out_projection()``  (tensor name, columns): the weight ``[hidden, columns]`` applied to what
+                          ``core`` leaves.
+    ``own_specs()`` / ``load_own(tensors, rt)``: every other tensor of the part.
+    ``core(ctx, proj, act, cache)``: ``proj[name]`` are the projected rows ``[T, rows]`` (columns of
+                          a wider buffer: unit column stride, any row stride), ``act [T, columns]``
+                          is to be filled.
+    """
+
+    hidden_size: int = 0
+    is_mixer = False
+
+    def in_projections(self):
+        raise NotImplementedError
+
+    def out_projection(self):
+        raise NotImplementedError
+
+    def own_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+
+    def core(self, ctx, proj, act, cache) -> None:
+        raise NotImplementedError
+
+    # -- on its own ----------------------------------------------------------------
+    def _own_set(self) -> "ProjectionSet":
+        s = getattr(self, "_set", None)
+        if s is None:
+            s = self._set = ProjectionSet(self.hidden_size, [("", self)])
+        return s
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return self._own_set().param_specs()
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self._own_set().load(tensors, rt)
+
+    def forward(self, ctx, normed, cache=None):
+        s = self._own_set()
+        proj, act = s.project(ctx, normed)
+        self.core(ctx, s.views(0, proj), s.act_view(0, act), cache)
+        return s.output(ctx, act)
+
+
+def _up8(n: int) -> int:
+    return (n + 7) // 8 * 8
+
+
+class ProjectionSet:
+    """The stacked projections of one or more ``ProjectedPart`` that read the same rows: one
+    weight ``[sum of rows, hidden]`` in, one ``[hidden, sum of columns]`` out.  Every part's slice
+    starts at a multiple of eight columns (16 bytes in bfloat16), the gaps being rows and columns
+    of zeros."""
+
+    def __init__(self, hidden_size: int, members):
+        from .linear import Linear
+        self.hidden_size = int(hidden_size)
+        self.members = list(members)                     # [(prefix, part)]
+        self.in_slices, self.act_slices = [], []
+        n_in = n_act = 0
+        for _, part in self.members:
+            views = {}
+            for name, rows in part.in_projections():
+                views[name] = (n_in, int(rows))
+                n_in = _up8(n_in + int(rows))
+            self.in_slices.append(views)
+            _, cols = part.out_projection()
+            self.act_slices.append((n_act, int(cols)))
+            n_act = _up8(n_act + int(cols))
+        self.n_in, self.n_act = n_in, n_act
+        self.w_in = Linear(self.hidden_size, n_in)
+        self.w_out = Linear(n_act, self.hidden_size)
+        self._gaps = []                                  # columns of the activations nobody writes
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs: Dict[str, ParamSpec] = {}
+        for prefix, part in self.members:
+            for name, rows in part.in_projections():
+                specs[join_name(prefix, name)] = ParamSpec((int(rows), self.hidden_size))
+            name, cols = part.out_projection()
+            specs[join_name(prefix, name)] = ParamSpec((self.hidden_size, int(cols)))
+            for name, spec in part.own_specs().items():
+                specs[join_name(prefix, name)] = spec
+        return specs
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        w_in = torch.zeros((self.n_in, self.hidden_size), device=rt.device, dtype=rt.dtype)
+        w_out = torch.zeros((self.hidden_size, self.n_act), device=rt.device, dtype=rt.dtype)
+        self._gaps, end = [], 0
+        for (prefix, part), views, (a0, cols) in zip(self.members, self.in_slices, self.act_slices):
+            sub = narrow_tensors(tensors, prefix) if prefix else tensors
+            for name, (c0, rows) in views.items():
+                w_in[c0:c0 + rows] = sub[name].to(device=rt.device, dtype=rt.dtype)
+            w_out[:, a0:a0 + cols] = sub[part.out_projection()[0]].to(device=rt.device, dtype=rt.dtype)
+            if a0 > end:
+                self._gaps.append((end, a0))
+            end = a0 + cols
+            part.load_own(sub, rt)
+        if self.n_act > end:
+            self._gaps.append((end, self.n_act))
+        self.w_in.set_weight(w_in, rt)
+        self.w_out.set_weight(w_out, rt)
+
+    def project(self, ctx, normed):
+        """(projected rows [T, n_in], the buffer [T, n_act] the parts' ``core`` fill)."""
+        T = normed.shape[0]
+        proj = ctx.workspace.get("projset.in", T, self.n_in, self.rt.dtype)
+        self.w_in.forward(normed, proj)
+        act = ctx.workspace.get("projset.act", T, self.n_act, self.rt.dtype)
+        for a, b in self._gaps:                          # scratch may hold anything, and 0 * NaN is NaN
+            act[:, a:b].zero_()
+        return proj, act
+
+    def views(self, i: int, proj):
+        return {name: proj[:, c0:c0 + rows] for name, (c0, rows) in self.in_slices[i].items()}
+
+    def act_view(self, i: int, act):
+        a0, cols = self.act_slices[i]
+        return act[:, a0:a0 + cols]
+
+    def output(self, ctx, act):
+        """The parts' summed outputs as a delta for the residual stream: 32-bit, or a stack of
+        32-bit partial sums that the next norm adds up."""
+        return self.rt.ops.linear_delta(act, self.w_out.weight, ctx.workspace, "projset.out",
+                                        self.w_out.weight_tiled, out_dtype=torch.float32)

@@ -15,7 +15,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import FeedForward, Mixer, Norm, ParamSpec, Part, Runtime, narrow_tensors
+from .base import FeedForward, Mixer, Norm, ParamSpec, Part, ProjectionSet, Runtime, join_name, narrow_tensors
 
 
 class Hidden:
@@ -68,7 +68,7 @@ class PreNormBlock(Part):
         specs = {}
         for prefix, part in self._children():
             for name, spec in part.param_specs().items():
-                specs[f"{prefix}.{name}"] = spec
+                specs[join_name(prefix, name)] = spec
         return specs
 
     def load(self, tensors, rt: Runtime) -> None:
@@ -147,3 +147,71 @@ class PreNormBlock(Part):
                     hidden.pending, hidden.deferred = None, (norm, prepared)
                     return
         hidden.pending, hidden.deferred = part.forward(ctx, inp, *cache), None
+
+
+class ParallelBlock(Part):
+    """One norm, and a mixer and a feed-forward that both read it:
+    ``n = norm(x); x <- x + mixer(n) + ffn(n)``.  Either sub-layer may be absent.
+
+    Both sub-layers are ``ProjectedPart``: their input projections are one product of ``n``, their
+    output projections one product over the concatenated activations, whose result is the block's
+    one delta (left pending for the next norm, as in ``PreNormBlock``)."""
+
+    takes_follow = False
+
+    def __init__(self, hidden_size: int, norm: Norm, mixer=None, ffn=None, names: Optional[Dict[str, str]] = None):
+        if mixer is None and ffn is None:
+            raise ValueError("a block needs a mixer or a feed-forward")
+        self.hidden_size = int(hidden_size)
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+        self.names = {"norm": "norm", "mixer": "mixer", "ffn": "ffn"}
+        if names:
+            self.names.update(names)
+        members = [(self.names[key], part) for key, part in (("mixer", mixer), ("ffn", ffn)) if part is not None]
+        self.set = ProjectionSet(self.hidden_size, members)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = {join_name(self.names["norm"], n): s for n, s in self.norm.param_specs().items()}
+        specs.update(self.set.param_specs())
+        return specs
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.norm.load(narrow_tensors(tensors, self.names["norm"]), rt)
+        self.set.load(tensors, rt)
+
+    def cache_need(self):
+        return self.mixer.cache_need() if self.mixer is not None else None
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", True) for p in (self.norm, self.mixer, self.ffn) if p is not None)
+
+    def can_cut_rows(self) -> bool:
+        return False
+
+    def entry(self):
+        return (self.norm, None)
+
+    def _run(self, ctx, hidden: Hidden, cache, mixer_only: bool):
+        normed = ctx.workspace.get("block.normed", hidden.x.shape[0], self.hidden_size, self.rt.dtype)
+        inp = hidden.input_behind(ctx, self.norm, normed)
+        proj, act = self.set.project(ctx, inp)
+        i = 0
+        if self.mixer is not None:
+            self.mixer.core(ctx, self.set.views(0, proj), self.set.act_view(0, act), cache)
+            i = 1
+        if mixer_only:
+            return None
+        if self.ffn is not None:
+            self.ffn.core(ctx, self.set.views(i, proj), self.set.act_view(i, act), None)
+        return self.set.output(ctx, act)
+
+    def forward(self, ctx, hidden: Hidden, cache, out_rows=None, follow=None) -> None:
+        hidden.pending, hidden.deferred = self._run(ctx, hidden, cache, False), None
+
+    def update_cache_only(self, ctx, hidden: Hidden, cache) -> None:
+        """The last block of a step whose logits nobody wants: the mixer alone runs, for what it
+        leaves in its cache or state; ``hidden`` is not meaningful afterwards."""
+        if self.mixer is not None:
+            self._run(ctx, hidden, cache, True)

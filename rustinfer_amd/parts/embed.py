@@ -15,17 +15,18 @@ from .base import ParamSpec, Part, Runtime, split_normed, stored_to
 
 
 class Embedding(Part):
-    def __init__(self, vocab_size: int, dim: int):
+    def __init__(self, vocab_size: int, dim: int, weight_name: str = "weight"):
         self.vocab_size = int(vocab_size)
         self.dim = int(dim)
         self.weight = None
+        self.weight_name = weight_name       # "" where the table carries the part's own name
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.vocab_size, self.dim), "matrix")}
+        return {self.weight_name: ParamSpec((self.vocab_size, self.dim), "matrix")}
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = stored_to(tensors["weight"], rt)
+        self.weight = stored_to(tensors[self.weight_name], rt)
 
     def forward(self, ctx, ids: torch.Tensor, out_x: torch.Tensor) -> torch.Tensor:
         self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None))
@@ -33,11 +34,15 @@ class Embedding(Part):
 
 
 class LMHead(Part):
-    def __init__(self, vocab_size: int, dim: int, tied_to: Optional[Embedding] = None):
+    def __init__(self, vocab_size: int, dim: int, tied_to: Optional[Embedding] = None,
+                 logit_scale: float = 1.0, softcap: float = 0.0):
+        """``logit_scale``, ``softcap``: the logits leave as ``softcap * tanh(logit_scale * z / softcap)``
+        (``softcap = 0``: ``logit_scale * z``)."""
         self.vocab_size = int(vocab_size)
         self.dim = int(dim)
         self.tied_to = tied_to
         self.weight = None
+        self.logit_scale, self.softcap = float(logit_scale), float(softcap)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         if self.tied_to is not None:
@@ -60,4 +65,6 @@ class LMHead(Part):
             self.rt.ops.linear(rows, self.weight, logits, self.weight_tiled)
         else:
             self.rt.ops.linear(rows, self.weight, logits, self.weight_tiled, scale=scale)
+        if self.logit_scale != 1.0 or self.softcap > 0.0:
+            self.rt.ops.scale_softcap(logits, self.logit_scale, self.softcap)
         return logits

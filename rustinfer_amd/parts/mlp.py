@@ -11,7 +11,7 @@ from typing import Dict
 
 import torch
 
-from .base import DeferredNorm, FeedForward, ParamSpec, Runtime, split_normed
+from .base import DeferredNorm, FeedForward, ParamSpec, ProjectedPart, Runtime, split_normed
 from .linear import Linear
 
 
@@ -70,3 +70,27 @@ class SwiGLUMLP(FeedForward):
         a, ssq = ops.linear_residual(act, self.down.weight, self.down.weight_tiled, x, next_norm.weight,
                                      ctx.workspace, "deferred")
         return DeferredNorm(a, ssq, next_norm.eps)
+
+
+class DenseMLP(ProjectedPart, FeedForward):
+    """``down(f(up(x)))`` with an elementwise ``f`` of the kernels' list (``relu2``: the square of
+    relu; ``tanh``).  Tensors ``up [ff, hidden]`` and ``down [hidden, ff]`` under the given names."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2",
+                 up_name: str = "up", down_name: str = "down"):
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.activation = activation
+        self.up_name, self.down_name = up_name, down_name
+
+    def in_projections(self):
+        return [(self.up_name, self.intermediate_size)]
+
+    def out_projection(self):
+        return (self.down_name, self.intermediate_size)
+
+    def core(self, ctx, proj, act, cache=None) -> None:
+        self.rt.ops.unary(self.activation, proj[self.up_name], act)
+
+    def forward(self, ctx, normed):
+        return ProjectedPart.forward(self, ctx, normed, None)

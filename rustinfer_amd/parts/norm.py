@@ -17,17 +17,20 @@ from .base import Norm, ParamSpec, Runtime, stored_to
 
 
 class RMSNorm(Norm):
-    def __init__(self, dim: int, eps: float):
+    def __init__(self, dim: int, eps: float, weight_name: str = "weight"):
+        """``weight_name``: the weight's name under the norm's own ("" where the tensor carries the
+        norm's name itself)."""
         self.dim = int(dim)
         self.eps = float(eps)
         self.weight = None
+        self.weight_name = weight_name
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.dim,), "norm")}
+        return {self.weight_name: ParamSpec((self.dim,), "norm")}
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = stored_to(tensors["weight"], rt, keep_fp32=True)
+        self.weight = stored_to(tensors[self.weight_name], rt, keep_fp32=True)
 
     cuts_rows = True          # forward() takes x_rows (see PreNormBlock.forward)
     # nothing but ``weight`` and ``eps``: the sub-layers around this norm may do it between them

@@ -1,0 +1,123 @@
+"""Mixers that keep a matrix of state for each head instead of a cache of keys.
+
+Both walk a request's tokens in order through ``S [key rows, value columns]`` (32-bit, in the
+request's state slot, zeros before its first token):
+
+``LightningAttention``   ``S <- decay_h S + k v^T``, ``o = S^T q`` with q, k, v = silu of their
+                         projections and one fixed decay for each head; the heads' outputs are
+                         normalised together (RMS over all of them, a learned weight), gated by
+                         ``sigmoid(W_g x)`` and projected.
+``GeneralDeltaRule``     ``S <- diag(w) S - (a u)(u^T S) + k v^T``, ``o = S^T r``: ``u`` the key of
+                         unit length, ``w = exp(-c sigmoid(W_w2 tanh(W_w1 x) + w0))`` a decay and
+                         ``a = sigmoid(W_a x + b_a)`` a removal rate for each key channel (both
+                         terms read the old state); each head's output is divided by its own root
+                         mean square, then a learned weight, the gate and the projection.
+
+The walk is one kernel for prompt portions and single tokens alike (``csrc/recurrent.hip``);
+everything between the projections and the gated norm's output is 32-bit.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from .base import Mixer, ParamSpec, ProjectedPart, Runtime, StateNeed
+from .linear import Linear
+
+
+class LightningAttention(ProjectedPart, Mixer):
+    is_mixer = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, decay: Sequence[float],
+                 norm_eps: float, names: Optional[Dict[str, str]] = None):
+        if len(decay) != num_heads:
+            raise ValueError(f"{len(decay)} decays for {num_heads} heads")
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.head_dim, self.v_head_dim = int(num_heads), int(head_dim), int(v_head_dim)
+        self.decay_values = [float(x) for x in decay]
+        self.norm_eps = float(norm_eps)
+        self.names = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm"}
+        if names:
+            self.names.update(names)
+
+    def in_projections(self):
+        n, hk, hv = self.names, self.num_heads * self.head_dim, self.num_heads * self.v_head_dim
+        return [(n["q"], hk), (n["k"], hk), (n["v"], hv), (n["g"], hv)]
+
+    def out_projection(self):
+        return (self.names["o"], self.num_heads * self.v_head_dim)
+
+    def own_specs(self):
+        return {self.names["norm"]: ParamSpec((self.num_heads * self.v_head_dim,), "norm")}
+
+    def cache_need(self):
+        return StateNeed((self.num_heads, self.head_dim, self.v_head_dim), torch.float32)
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.norm_weight = tensors[self.names["norm"]].to(device=rt.device, dtype=torch.float32).contiguous()
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=rt.device)
+
+    def core(self, ctx, proj, act, cache) -> None:
+        ops, n = self.rt.ops, self.names
+        T = act.shape[0]
+        o = ctx.workspace.get("scan.o", T, self.num_heads * self.v_head_dim, torch.float32)
+        ops.linear_scan(proj[n["q"]], proj[n["k"]], proj[n["v"]], cache.state, o, ctx, self.num_heads,
+                        self.head_dim, self.v_head_dim, decay=self.decay, silu_in=True)
+        ops.gated_group_norm(o, self.norm_weight, proj[n["g"]], act, self.num_heads * self.v_head_dim, self.norm_eps)
+
+
+class GeneralDeltaRule(ProjectedPart, Mixer):
+    is_mixer = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, decay_rank: int, norm_eps: float,
+                 decay_strength: float = math.exp(-0.5), unit_eps: float = 1e-6,
+                 names: Optional[Dict[str, str]] = None):
+        """``decay_rank``: rows of the first of the two matrices that make the decay's input;
+        ``decay_strength``: the ``c`` of ``w = exp(-c sigmoid(.))``, so that ``w`` stays in
+        ``(exp(-c), 1)``; ``unit_eps``: added to ``|k|^2`` under the root of the unit key."""
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.head_dim, self.decay_rank = int(num_heads), int(head_dim), int(decay_rank)
+        self.norm_eps, self.decay_strength, self.unit_eps = float(norm_eps), float(decay_strength), float(unit_eps)
+        self.names = {"r": "r", "k": "k", "v": "v", "g": "g", "a": "a", "a_bias": "a.b", "w1": "w1", "w2": "w2",
+                      "w0": "w0", "o": "o", "norm": "norm"}
+        if names:
+            self.names.update(names)
+        self.w2 = Linear(self.decay_rank, self.num_heads * self.head_dim)
+
+    def in_projections(self):
+        n, hd = self.names, self.num_heads * self.head_dim
+        return [(n["r"], hd), (n["k"], hd), (n["v"], hd), (n["g"], hd), (n["a"], hd), (n["w1"], self.decay_rank)]
+
+    def out_projection(self):
+        return (self.names["o"], self.num_heads * self.head_dim)
+
+    def own_specs(self):
+        n, hd = self.names, self.num_heads * self.head_dim
+        return {n["w2"]: ParamSpec((hd, self.decay_rank)), n["w0"]: ParamSpec((hd,), mean=0.0, std=1.0),
+                n["a_bias"]: ParamSpec((hd,), mean=0.0, std=1.0), n["norm"]: ParamSpec((hd,), "norm")}
+
+    def cache_need(self):
+        return StateNeed((self.num_heads, self.head_dim, self.head_dim), torch.float32)
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        n = self.names
+        f32 = lambda name: tensors[name].to(device=rt.device, dtype=torch.float32).contiguous()
+        self.w0, self.a_bias, self.norm_weight = f32(n["w0"]), f32(n["a_bias"]), f32(n["norm"])
+        self.w2.set_weight(tensors[n["w2"]], rt)
+
+    def core(self, ctx, proj, act, cache) -> None:
+        ops, n = self.rt.ops, self.names
+        T, hd = act.shape[0], self.num_heads * self.head_dim
+        w1 = proj[n["w1"]]
+        ops.unary("tanh", w1, w1)
+        wl = ctx.workspace.get("gdr.wl", T, hd, self.rt.dtype)
+        self.w2.forward(w1, wl)
+        o = ctx.workspace.get("scan.o", T, hd, torch.float32)
+        ops.linear_scan(proj[n["r"]], proj[n["k"]], proj[n["v"]], cache.state, o, ctx, self.num_heads,
+                        self.head_dim, self.head_dim, wl=wl, al=proj[n["a"]], w0=self.w0, ab=self.a_bias,
+                        unit_eps=self.unit_eps, decay_c=self.decay_strength)
+        ops.gated_group_norm(o, self.norm_weight, proj[n["g"]], act, self.head_dim, self.norm_eps)

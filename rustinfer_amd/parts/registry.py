@@ -4,13 +4,15 @@ from __future__ import annotations
 
 from typing import Callable, Dict
 
-from .attention import PagedAttention
-from .mlp import SwiGLUMLP
+from .attention import PagedAttention, WindowAttention
+from .mlp import DenseMLP, SwiGLUMLP
 from .norm import RMSNorm
+from .recurrent import GeneralDeltaRule, LightningAttention
 from .rope import RotaryEmbedding
 
-MIXERS: Dict[str, Callable] = {"attention": PagedAttention}
-FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP}
+MIXERS: Dict[str, Callable] = {"attention": PagedAttention, "window_attention": WindowAttention,
+                               "lightning": LightningAttention, "general_delta": GeneralDeltaRule}
+FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP, "dense": DenseMLP}
 NORMS: Dict[str, Callable] = {"rmsnorm": RMSNorm}
 POSITION_ENCODINGS: Dict[str, Callable] = {"rope": RotaryEmbedding}
 
