@@ -105,7 +105,7 @@ class LLM:
         notes = set()
         for layer in getattr(self.engine.model, "layers", ()) if why is not None else ():
             m = getattr(layer, "mixer", None)
-            if all(hasattr(m, a) for a in ("num_heads", "num_kv_heads", "head_dim")):
+            if all(hasattr(m, a) for a in ("num_heads", "num_kv_heads", "head_dim")) and not hasattr(m, "v_head_dim"):
                 note = why(self.engine.rt.dtype, m.num_heads, m.num_kv_heads, m.head_dim, self.engine.page_size)
                 if note:
                     notes.add(note)
