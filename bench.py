@@ -317,6 +317,127 @@ class Bench:
         self.torch.cuda.empty_cache()
 
 
+# Tedelix at the layer sizes of the Llama shapes: the same width, feed-forward width, number of
+# layers and heads; its three mixers take turns; windows of 1,024 positions.
+TEDELIX_PATTERN = ("general_delta", "attention", "lightning")
+
+
+def tedelix_config(shape_name, layers=0, window=1024):
+    s = SHAPES[shape_name]
+    H, G, hd, W = s["num_attention_heads"], s["num_key_value_heads"], s["head_dim"], s["hidden_size"]
+    out = []
+    for i in range(layers or s["num_hidden_layers"]):
+        kind = TEDELIX_PATTERN[i % len(TEDELIX_PATTERN)]
+        if kind == "attention":
+            mixer = dict(heads=H, kv_heads=G, dim=hd, vdim=hd, mask=dict(size=window), scale=hd ** -0.5,
+                         rot=dict(base=10000.0, dims=hd))
+        elif kind == "lightning":
+            mixer = dict(heads=H, dim=hd, vdim=hd, decay=[1.0 - 2.0 ** (-5 - 3 * h / max(H - 1, 1)) for h in range(H)])
+        else:
+            mixer = dict(heads=H, dim=hd)
+        out.append(dict(type=kind, mixer=mixer, mlp=dict(kind="dense", ff=s["intermediate_size"])))
+    return dict(architecture="Tedelix", vocab=s["vocab_size"], width=W, norm=dict(eps=1e-6), logit_scale=1.0,
+                logit_softcap=30.0, layers=out)
+
+
+class TedelixBench(Bench):
+    """The same measurements on a Tedelix model of a Llama shape's sizes."""
+
+    def __init__(self, shape_name, args, max_batch):
+        import torch
+        from rustinfer_amd.llm import LLM
+        self.torch, self.args = torch, args
+        self.window = 1024
+        conf = tedelix_config(shape_name, args.layers, self.window)
+        self.full_layers = SHAPES[shape_name]["num_hidden_layers"]
+        self.prompt_len = args.context // 2
+        self.dir = tempfile.TemporaryDirectory()
+        with open(os.path.join(self.dir.name, "config.json"), "w") as f:
+            json.dump(conf, f)
+        self.llm = LLM(model=self.dir.name, random_weights_seed=0, dtype="bfloat16" if args.dtype == "bf16" else "float32",
+                       paged_block_size=PAGE, num_blocks=max_batch * (args.context // PAGE) + 8, max_batch_seqs=max_batch,
+                       max_model_len=args.context, max_batch_tokens=max(8192, self.prompt_len),
+                       capture_sizes=sorted({1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, args.batch}),
+                       gemm_tune=not args.no_gemm_tune, step_token_align=0 if getattr(args, "no_token_align", False) else 256)
+        self.engine = self.llm.engine
+        if args.no_graph:
+            self.engine.enable_graphs(False)
+        self.cfg = cfg = self.llm.model_config
+        el = 2 if args.dtype == "bf16" else 4
+        self.params = 0
+        for name, spec in self.engine.model.param_specs().items():
+            n = 1
+            for d in spec.shape:
+                n *= int(d)
+            self.params += n
+        self.weight_bytes = el * self.params
+        # what a decoding request reads a step beside the weights: the keys and values inside its
+        # windows, and its states (read and written back, 32-bit)
+        self.window_kv_bytes = self.state_bytes = 0
+        self.attn_flops_per_key = self.scan_flops_per_token = 0
+        for layer in cfg.layers:
+            m = layer.mixer
+            if layer.type == "attention":
+                self.window_kv_bytes += m.kv_heads * (m.dim + m.vdim) * el
+                self.attn_flops_per_key += 2.0 * m.heads * (m.dim + m.vdim)
+            elif layer.type == "lightning":
+                self.state_bytes += 2 * 4 * m.heads * m.dim * m.vdim
+                self.scan_flops_per_token += 2.0 * 2 * m.heads * m.dim * m.vdim
+            else:
+                self.state_bytes += 2 * 4 * m.heads * m.dim * m.dim
+                self.scan_flops_per_token += 2.0 * 5 * m.heads * m.dim * m.dim
+        self.gen = torch.Generator(device="cuda").manual_seed(1)
+
+    @property
+    def kv_bytes_per_token(self):          # Bench.decode prices a step as weights + batch * context * this
+        ctx = self.prompt_len + 64
+        return (min(ctx, self.window) * self.window_kv_bytes + self.state_bytes) / ctx
+
+    def prefill(self, tokens_n=2048, reps=5):
+        from rustinfer_amd.engine import StepEntry
+        torch, cfg = self.torch, self.cfg
+        self.release_all()
+        ids = self.random_ids(tokens_n)
+        times = []
+        for r in range(reps + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            self.engine.step([StepEntry("p", ids, [tokens_n - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            self.engine.release("p")
+        t = sorted(times[1:])[len(times[1:]) // 2]
+        keys = sum(min(i + 1, self.window) for i in range(tokens_n))
+        products = 2.0 * tokens_n * (self.params - cfg.vocab_size * cfg.hidden_size) + 2.0 * cfg.vocab_size * cfg.hidden_size
+        mixers = self.attn_flops_per_key * keys + self.scan_flops_per_token * tokens_n
+        return {"value": round(tokens_n / t, 1), "tokens": tokens_n, "ms": round(t * 1e3, 3),
+                "frac": round((products + mixers) / t / PEAK_FLOPS[self.args.dtype], 4),
+                "product_flops": products, "mixer_flops_32bit": mixers}
+
+
+def design_record(args, peaks):
+    """``--design tedelix``: decode at the main batch and prefill of 2,048 tokens for Tedelix models of
+    the sizes of ``--design-shapes``, each beside the Llama model of the same sizes."""
+    out = {"metric": "decode tok/s at batch %d and prefill tok/s at 2,048 tokens: Tedelix beside Llama at equal layer sizes" % args.batch,
+           "unit": "tok/s", "dtype": args.dtype, "data": "synthetic: random weights, random token ids", "peaks": peaks,
+           "pattern": list(TEDELIX_PATTERN), "window": 1024, "shapes": {}}
+    steps = max(MIN_POINT_STEPS, args.steps)
+    for name in args.design_shapes.split(","):
+        rec = {}
+        for who, cls in (("tedelix", TedelixBench), ("llama", Bench)):
+            if who == "llama" and args.no_points:
+                continue
+            b = cls(name, args, args.batch)
+            tok_s, step_s, step_bytes = b.decode(args.batch, steps, args.warmup)
+            gbs = step_bytes / step_s / 1e9
+            rec[who] = {"decode": round(tok_s, 1), "ms_per_step": round(step_s * 1e3, 4), "layers": len(b.engine.model.layers),
+                        "decode_bytes_a_step": int(step_bytes), "roofline_frac": round(gbs / PEAK_HBM_GBS, 4),
+                        "prefill": b.prefill(reps=3)}
+            b.close()
+        out["shapes"][name] = rec
+    return out
+
+
 def other_shape(name, args, dtype, peaks):
     """Decode at the main batch and prefill of another shape or precision, as a sub-record."""
     sub = argparse.Namespace(**vars(args))
@@ -395,6 +516,10 @@ def main() -> int:
                     help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",
                     help="keep the GEMM library's own choice of kernel for the prompt's products")
+    ap.add_argument("--design", default="llama", choices=["llama", "tedelix"],
+                    help="tedelix: only decode and prefill of Tedelix models at the sizes of --design-shapes, each beside "
+                         "the Llama model of the same sizes (the default workload is not run)")
+    ap.add_argument("--design-shapes", default="1b,3b", help="shapes for --design tedelix, with commas between them")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -405,6 +530,9 @@ def main() -> int:
         print(json.dumps(sampling_times(ops, SHAPES[args.shape]["vocab_size"], args.steps)))
         return 0
     peaks = ops.measure_peaks()
+    if args.design == "tedelix":
+        print(json.dumps(design_record(args, peaks)))
+        return 0
     b = Bench(args.shape, args, max(args.batch, 16 if args.mixed else 1 if (args.no_points or args.prompt) else 64))
     cfg = b.cfg
     if args.no_mixed_graph:

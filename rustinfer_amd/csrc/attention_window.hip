@@ -114,13 +114,29 @@ __device__ __forceinline__ void aw_merge(float& m, float& l, float (&acc)[NC], f
     m = M;
 }
 
+// 16 bytes of the cache as 32-bit values: 4 floats or 8 bfloat16
+__device__ __forceinline__ void ld_vec16(const float* p, float* f) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+__device__ __forceinline__ void ld_vec16(const bf16_t* p, float* f) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+    f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+    f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
 template <typename T, int NC>    // NC: 64-wide slices of the value head a lane holds
 __global__ __launch_bounds__(256) void attn_window_kernel(
         const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
         const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window, int TQ, int NK,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved,
+        int slots, float* __restrict__ part_ml, float* __restrict__ part_o) {
+    // slots > 0 (steps of single tokens): the block takes ONE block of keys, the blockIdx.z-th of
+    // its row's window, and leaves its partial result for attn_window_combine_kernel
     extern __shared__ __align__(16) float lds[];
     const int dkp = (dk + 3) & ~3, ks_stride = dkp + 4, vs_stride = dv + 1;
     float* Qs = lds;                                   // [AW_ROWS][dkp]
@@ -168,7 +184,13 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
         row_lo[i] = window > 0 ? max(0, p + 1 - window) : 0;
     }
 
-    for (int kb = first_key / NK; kb * NK < last_visible; ++kb) {
+    int kb_lo = first_key / NK, kb_hi = (last_visible + NK - 1) / NK;
+    if (slots > 0) {
+        kb_lo += blockIdx.z;
+        kb_hi = min(kb_hi, kb_lo + 1);
+        if (kb_lo >= kb_hi) return;                    // the row's window has fewer blocks of keys
+    }
+    for (int kb = kb_lo; kb < kb_hi; ++kb) {
         const int j_base = kb * NK;
         __syncthreads();                               // the last block of keys has been used (first pass: Qs is written)
         if (tid < NK) {
@@ -181,11 +203,45 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
             koff[tid] = off;
         }
         __syncthreads();
-        for (int e = tid; e < NK * dkp; e += 256) {
-            const int jj = e / dkp, dd = e - jj * dkp, off = koff[jj];
-            Ks[jj * ks_stride + dd] = (off >= 0 && dd < dk) ? ld_f32(kc + (size_t)off * dk + dd) : 0.f;
+        constexpr int VL = 16 / sizeof(T);              // elements of a 16-byte load
+        if (dk % VL == 0) {                            // keys: 16 bytes a thread and load
+            const int pieces = dk / VL;
+            for (int e = tid; e < NK * pieces; e += 256) {
+                const int jj = e / pieces, pc = e - jj * pieces, off = koff[jj];
+                float f[VL];
+#pragma unroll
+                for (int u = 0; u < VL; ++u) f[u] = 0.f;
+                if (off >= 0) ld_vec16(kc + (size_t)off * dk + pc * VL, f);
+#pragma unroll
+                for (int u = 0; u < VL; u += 4)
+                    *reinterpret_cast<float4*>(Ks + jj * ks_stride + pc * VL + u) = make_float4(f[u], f[u + 1], f[u + 2], f[u + 3]);
+            }
+        } else {
+            for (int e = tid; e < NK * dkp; e += 256) {
+                const int jj = e / dkp, dd = e - jj * dkp, off = koff[jj];
+                Ks[jj * ks_stride + dd] = (off >= 0 && dd < dk) ? ld_f32(kc + (size_t)off * dk + dd) : 0.f;
+            }
         }
-        {
+        if (page % VL == 0) {
+            // values: the positions of a feature are contiguous; VL of them (inside one page,
+            // since blocks of keys and pages both start at multiples of VL) a thread and load
+            const int runs = NK / VL;
+            for (int e = tid; e < runs * dv; e += 256) {
+                const int d = e / runs, jj0 = (e - d * runs) * VL;
+                float f[VL];
+#pragma unroll
+                for (int u = 0; u < VL; ++u) f[u] = 0.f;
+                int first = -1;
+#pragma unroll
+                for (int u = 0; u < VL; ++u) if (first < 0 && koff[jj0 + u] >= 0) first = u;
+                if (first >= 0) {
+                    const int off = koff[jj0 + first] - first;           // slot of the run's first position
+                    ld_vec16(vc + (size_t)(off / page) * page * dv + (size_t)d * page + off % page, f);
+                }
+#pragma unroll
+                for (int u = 0; u < VL; ++u) Vs[(jj0 + u) * vs_stride + d] = koff[jj0 + u] >= 0 ? f[u] : 0.f;
+            }
+        } else {
             const int jj = tid % NK, off = koff[jj];
             const size_t vbase = off >= 0 ? (size_t)(off / page) * page * dv + off % page : 0;
             for (int d = tid / NK; d < dv; d += 256 / NK)
@@ -254,6 +310,21 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) aw_merge<NC>(m[i], l[i], acc[i], m_b[i], l_b[i], acc_b[i]);
     }
+    if (slots > 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = wave + 4 * i;
+            if (r >= R) continue;
+            const size_t at = ((size_t)(t0 + r / G) * H + (g * G + r % G)) * slots + blockIdx.z;
+            if (lane == 0) { part_ml[at * 2] = m[i]; part_ml[at * 2 + 1] = l[i]; }
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const int d = lane + 64 * c;
+                if (d < dv) part_o[at * dv + d] = acc[i][c];
+            }
+        }
+        return;
+    }
     if (vcos == nullptr) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -296,6 +367,60 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
     }
 }
 
+// Steps of single tokens: merge the partial results of a row's blocks of keys in ascending order
+// (the order and the arithmetic of the loop in attn_window_kernel, so a token's output has the
+// same bits as there), divide, turn back, write.  One wave a (token, head).
+template <typename T, int NC>
+__global__ __launch_bounds__(64) void attn_window_combine_kernel(
+        const float* __restrict__ part_ml, const float* __restrict__ part_o, T* __restrict__ out, int out_stride,
+        const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
+        int H, int dv, int window, int NK, int slots,
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+    __shared__ float Os[256];
+    const int b = blockIdx.y, h = blockIdx.x, lane = threadIdx.x;
+    const int t = cu_q[b];
+    if (cu_q[b + 1] - t <= 0) return;                  // a row without a token
+    const int p = q_start[b];
+    const int visible = min(kv_lens[b], p + 1);
+    const int first_key = window > 0 ? max(0, p + 1 - window) : 0;
+    const int n = (visible + NK - 1) / NK - first_key / NK;
+    float m = -INFINITY, l = 0.f, acc[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[c] = 0.f;
+    for (int s = 0; s < n && s < slots; ++s) {
+        const size_t at = ((size_t)t * H + h) * slots + s;
+        float acc_b[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int d = lane + 64 * c;
+            acc_b[c] = d < dv ? part_o[at * dv + d] : 0.f;
+        }
+        aw_merge<NC>(m, l, acc, part_ml[at * 2], part_ml[at * 2 + 1], acc_b);
+    }
+    T* o = out + (size_t)t * out_stride + h * dv;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int d = lane + 64 * c;
+        if (d < dv) {
+            const float y = l > 0.f ? acc[c] / l : 0.f;
+            if (vcos == nullptr) st_f32(o + d, y);
+            else Os[d] = y;
+        }
+    }
+    if (vcos == nullptr) return;
+    __syncthreads();
+    const int vh = dv >> 1;
+    for (int mm = lane; mm < vh; mm += 64) {
+        const int i0 = v_interleaved ? 2 * mm : mm, i1 = v_interleaved ? 2 * mm + 1 : mm + vh;
+        const float a = Os[i0], bb = Os[i1];
+        const float c = vcos[(size_t)p * vh + mm], s = vsin[(size_t)p * vh + mm];
+        st_f32(o + i0, a * c + bb * s);
+        st_f32(o + i1, bb * c - a * s);
+    }
+}
+
+int aw_keys_a_block(int dk, int dv);
+
 size_t aw_lds_bytes(int dk, int dv, int NK) {
     const int dkp = (dk + 3) & ~3;
     const size_t kv = (size_t)NK * (dkp + 4) + (size_t)NK * (dv + 1);
@@ -304,6 +429,19 @@ size_t aw_lds_bytes(int dk, int dv, int NK) {
 }
 
 constexpr size_t AW_LDS_MOST = 150 * 1024;
+
+int aw_keys_a_block(int dk, int dv) {
+    int NK = 64;
+    while (NK > 16 && aw_lds_bytes(dk, dv, NK) > AW_LDS_MOST) NK >>= 1;
+    return NK;
+}
+
+// blocks of keys the window of a single token can touch when no request is longer than max_kv_len
+int aw_slots(int dk, int dv, int window, int max_kv_len) {
+    const int NK = aw_keys_a_block(dk, dv);
+    const int span = window > 0 ? min(window, max_kv_len) : max_kv_len;
+    return (span + NK - 1) / NK + (window > 0 ? 1 : 0);      // a window may begin inside a block: one more
+}
 
 }  // namespace
 
@@ -340,10 +478,10 @@ namespace {
 template <typename T>
 int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
               const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
-              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, hipStream_t stream) {
+              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved,
+              int slots, float* workspace, hipStream_t stream) {
     const int G = H / Hkv, TQ = AW_ROWS / G;
-    int NK = 64;
-    while (NK > 16 && aw_lds_bytes(dk, dv, NK) > AW_LDS_MOST) NK >>= 1;
+    const int NK = aw_keys_a_block(dk, dv);
     const size_t lds = aw_lds_bytes(dk, dv, NK);
     const int NC = (dv + 63) / 64;
     auto kernel = NC == 1 ? attn_window_kernel<T, 1> : NC == 2 ? attn_window_kernel<T, 2> : NC == 3 ? attn_window_kernel<T, 3> : attn_window_kernel<T, 4>;
@@ -356,21 +494,45 @@ int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, con
             asked[NC] = true;
         }
     }
+    if (slots > 0) {
+        // every row has at most one token: a tile a row, a block a block of keys, then the merge
+        float* part_ml = workspace;
+        float* part_o = workspace + (size_t)Tn * H * slots * 2;
+        kernel<<<dim3(num_rows, Hkv, slots), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start,
+                                                              kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin,
+                                                              v_interleaved, slots, part_ml, part_o);
+        auto combine = NC == 1 ? attn_window_combine_kernel<T, 1> : NC == 2 ? attn_window_combine_kernel<T, 2>
+                     : NC == 3 ? attn_window_combine_kernel<T, 3> : attn_window_combine_kernel<T, 4>;
+        combine<<<dim3(H, num_rows), 64, 0, stream>>>(part_ml, part_o, out, out_stride, cu_q, q_start, kv_lens, H, dv, window, NK, slots,
+                                                      vcos, vsin, v_interleaved);
+        return 0;
+    }
     const int tiles = (Tn + TQ - 1) / TQ + num_rows;   // at most: every request may end in a short tile
     kernel<<<dim3(tiles, Hkv), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens,
-                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved);
+                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved,
+                                                   0, nullptr, nullptr);
     return 0;
 }
 }  // namespace
 
+// Floats of workspace for a step of T single tokens whose longest request has max_kv_len keys
+// (0: such a step has one block of keys a row at most and needs none).
+extern "C" size_t ri_attention_window_workspace(int T, int H, int dk, int dv, int window, int max_kv_len) {
+    const int slots = aw_slots(dk, dv, window, max_kv_len);
+    return slots <= 1 ? 0 : (size_t)T * H * slots * (dv + 2);
+}
+
 // Attention of the step's tokens (rotated queries in q) over the cache; out [T][>= H dv].
 // vcos / vsin [positions][dv / 2]: the sums are turned back by the query's position (null: not).
+// single_tokens != 0: every row of the step has at most one token and row b's token is token
+// cu_q[b]; with a workspace of ri_attention_window_workspace floats the keys of a row are then
+// divided between blocks (the same bits as without).
 extern "C" int ri_attention_window(
         const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kc, const void* vc,
         int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
         const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
         float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
-        hipStream_t stream) {
+        int single_tokens, int max_kv_len, float* workspace, size_t workspace_floats, hipStream_t stream) {
     RI_REQUIRE(ri_attention_window_supported(H, Hkv, dk, dv), "ri_attention_window: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
     RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window: bad sizes");
     RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window: row strides too small");
@@ -378,11 +540,18 @@ extern "C" int ri_attention_window(
     if (T == 0 || num_rows == 0) return 0;
     RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_window: null pointer");
     RI_REQUIRE(Hkv <= 65535, "ri_attention_window: too many key/value heads for the grid");
+    int slots = 0;
+    if (single_tokens && workspace && max_kv_len > 0) {
+        slots = aw_slots(dk, dv, window, max_kv_len);
+        if (slots <= 1) slots = 0;
+        else RI_REQUIRE(workspace_floats >= (size_t)T * H * slots * (dv + 2) && slots <= 65535 && num_rows <= 65535 && H <= 65535,
+                        "ri_attention_window: workspace of %zu floats for %d slots, or too many rows for the grid", workspace_floats, slots);
+    }
     int rc;
     if (dtype == RI_F32)
-        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, stream);
     else if (dtype == RI_BF16)
-        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, stream);
     else
         return ri_fail("ri_attention_window: unknown dtype %d", dtype);
     if (rc) return rc;

@@ -11,11 +11,13 @@
 // Both terms of the delta form read the old state.  Everything after the projections is 32-bit.
 //
 // One kernel walks a request's tokens of the step in order; a step of single tokens is the same
-// walk of one token.  A thread keeps 32 key rows of one value column in registers; the P threads
-// that share a column (P = the power of two with 32 P >= dk) sit in one wave, 64 / P lanes apart,
-// and add their partial dot products with lane exchanges.  The vectors of a stretch of eight
-// tokens are brought into LDS, activated, by the whole block; the walk then reads them as
-// broadcasts.  What a token adds up, and in which order, does not depend on how the request was
+// walk of one token.  A thread keeps R = 8 key rows (16 beyond 128 of them) of one value column in
+// registers; the P threads that share a column (P = the power of two with R P >= dk, at most 16)
+// are neighbouring lanes and add their partial dot products with lane exchanges that stay in the
+// vector unit.  The walk is a chain from token to token and a request has only heads x columns x P
+// threads, so what counts is how few instructions a thread spends on a token: hence few rows a
+// thread.  The vectors of a stretch of eight tokens are asked for a stretch ahead, brought into one
+// of two LDS buffers already activated, and read by the walk as broadcasts.  What a token adds up, and in which order, does not depend on how the request was
 // cut into steps, so the state and the outputs have the same bits for every cut.
 // A block holds NW waves (64 NW / P columns); with few (request, head) pairs a wave a block, so
 // that the chip has blocks enough.
@@ -24,8 +26,8 @@
 
 namespace {
 
-constexpr int SC_R = 32;         // key rows a thread
 constexpr int SC_CH = 8;         // tokens a stretch
+constexpr int SC_EPL = 4;        // most key rows a lane stages for one token (64 lanes x 4 >= 256)
 
 struct ScanArgs {
     const void *r, *k, *v, *wl, *al;
@@ -42,101 +44,155 @@ struct ScanArgs {
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ __forceinline__ float siluf_(float z) { return z / (1.f + expf(-z)); }
 
-template <typename T, bool DELTA, int NW>
+// Sum over the P adjacent lanes that share a column (P a power of two up to 16), every lane
+// getting the same bits: exchanges inside a quad, between the quads of half a row, between the
+// halves of a row of 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float group_sum(float x, int P) {
+    if (P >= 2) x += dpp_f<0xB1>(x);                   // quad_perm [1, 0, 3, 2]
+    if (P >= 4) x += dpp_f<0x4E>(x);                   // quad_perm [2, 3, 0, 1]
+    if (P >= 8) x += dpp_f<0x141>(x);                  // row_half_mirror
+    if (P >= 16) x += dpp_f<0x140>(x);                 // row_mirror
+    return x;
+}
+
+template <typename T, bool DELTA, int R, int NW>
 __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) {
     extern __shared__ __align__(16) float lds[];
-    const int P = a.P, DKP = P * SC_R, dk = a.dk, dv = a.dv, H = a.H;
+    constexpr int TPW = SC_CH / NW;                    // tokens of a stretch a wave stages
+    constexpr int NA = DELTA ? 5 : 2;
+    const int P = a.P, DKP = P * R, dk = a.dk, dv = a.dv, H = a.H;
     const int CW = 64 / P, CPB = NW * CW;
-    float* rs = lds;                                   // [SC_CH][DKP]
-    float* ks = rs + SC_CH * DKP;
-    float* us = ks + SC_CH * DKP;                      // the delta form's three
-    float* aus = us + SC_CH * DKP;
-    float* ws = aus + SC_CH * DKP;
-    float* vs = DELTA ? ws + SC_CH * DKP : us;         // [SC_CH][CPB]
+    const int BUF = NA * SC_CH * DKP + SC_CH * CPB;    // floats of one of the two stretch buffers
     const int b = blockIdx.z, h = blockIdx.y;
     const int t_lo = a.cu_q[b], n = a.cu_q[b + 1] - t_lo;
     if (n <= 0) return;                                // a row without tokens (padding of a captured shape)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int pl = lane / CW, cl = lane - pl * CW;
+    const int pl = lane % P, cl = lane / P;            // the P lanes of a column are neighbours
     const int jc = wave * CW + cl, j = blockIdx.x * CPB + jc;
     const bool col_ok = j < dv;
     float* Sg = a.state + ((size_t)a.slots[b] * H + h) * (size_t)dk * dv;
     const bool fresh = a.q_start[b] == 0;              // a request's first tokens start from nothing
-    float S[SC_R];
+    float S[R];
 #pragma unroll
-    for (int ii = 0; ii < SC_R; ++ii) {
-        const int i = pl * SC_R + ii;
+    for (int ii = 0; ii < R; ++ii) {
+        const int i = pl * R + ii;
         S[ii] = (!fresh && col_ok && i < dk) ? Sg[(size_t)i * dv + j] : 0.f;
     }
     const float dec = DELTA ? 0.f : a.decay[h];
     const T* rp = (const T*)a.r; const T* kp = (const T*)a.k; const T* vp = (const T*)a.v;
     const T* wlp = (const T*)a.wl; const T* alp = (const T*)a.al;
-    for (int c0 = 0; c0 < n; c0 += SC_CH) {
+
+    // what this thread stages of a stretch: asked for a stretch ahead, so that the walk hides the wait
+    float raw_r[TPW][SC_EPL], raw_k[TPW][SC_EPL], raw_w[DELTA ? TPW : 1][SC_EPL], raw_a[DELTA ? TPW : 1][SC_EPL];
+    float raw_v[SC_CH];
+    auto ask = [&](int c0) {
         const int nc = min(SC_CH, n - c0);
-        __syncthreads();                               // the last stretch has been walked
-        for (int tt = wave; tt < nc; tt += NW) {
-            const size_t t = (size_t)(t_lo + c0 + tt);
-            if (DELTA) {
-                float kk[4], ssq = 0.f;                // DKP / 64 <= 4 values a lane
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = e * 64 + lane;
-                    kk[e] = (i < dk) ? ld_f32(kp + t * a.k_stride + h * dk + i) : 0.f;
-                    ssq = fmaf(kk[e], kk[e], ssq);
+        for (int i = 0; i < TPW; ++i) {
+            const int tt = wave + i * NW;
+#pragma unroll
+            for (int e = 0; e < SC_EPL; ++e) {
+                const int idx = e * 64 + lane;
+                const bool on = tt < nc && idx < dk;
+                const size_t t = (size_t)(t_lo + c0 + (on ? tt : 0));
+                const int c = h * dk + (on ? idx : 0);
+                raw_r[i][e] = on ? ld_f32(rp + t * a.r_stride + c) : 0.f;
+                raw_k[i][e] = on ? ld_f32(kp + t * a.k_stride + c) : 0.f;
+                if (DELTA) {
+                    raw_w[i][e] = on ? ld_f32(wlp + t * a.wl_stride + c) : 0.f;
+                    raw_a[i][e] = on ? ld_f32(alp + t * a.al_stride + c) : 0.f;
                 }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < SC_CH; ++e) {
+            const int x = e * (NW * 64) + tid;
+            const int tt = x / CPB, c = x - tt * CPB, jj = blockIdx.x * CPB + c;
+            raw_v[e] = (x < nc * CPB && jj < dv) ? ld_f32(vp + (size_t)(t_lo + c0 + tt) * a.v_stride + h * dv + jj) : 0.f;
+        }
+    };
+    auto stage = [&](float* buf, int nc) {
+        float* rs = buf;                               // [SC_CH][DKP] each
+        float* ks = rs + SC_CH * DKP;
+        float* us = ks + SC_CH * DKP;                  // the delta form's three
+        float* aus = us + SC_CH * DKP;
+        float* ws = aus + SC_CH * DKP;
+        float* vs = buf + NA * SC_CH * DKP;            // [SC_CH][CPB]
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int tt = wave + i * NW;
+            if (tt >= nc) continue;
+            if (DELTA) {
+                float ssq = 0.f;
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) ssq = fmaf(raw_k[i][e], raw_k[i][e], ssq);
                 ssq = wave_sum(ssq);
                 const float inv = 1.f / sqrtf(ssq + a.unit_eps);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = e * 64 + lane;
-                    if (i >= DKP) continue;
-                    float r = 0.f, u = 0.f, au = 0.f, w = 0.f;
-                    if (i < dk) {
-                        const int c = h * dk + i;
-                        r = ld_f32(rp + t * a.r_stride + c);
-                        u = kk[e] * inv;
-                        au = sigmoidf_(ld_f32(alp + t * a.al_stride + c) + a.ab[c]) * u;
-                        w = expf(-a.decay_c * sigmoidf_(ld_f32(wlp + t * a.wl_stride + c) + a.w0[c]));
+                for (int e = 0; e < SC_EPL; ++e) {
+                    const int idx = e * 64 + lane;
+                    if (idx >= DKP) continue;
+                    float u = 0.f, au = 0.f, w = 0.f;
+                    if (idx < dk) {
+                        const int c = h * dk + idx;
+                        u = raw_k[i][e] * inv;
+                        au = sigmoidf_(raw_a[i][e] + a.ab[c]) * u;
+                        w = expf(-a.decay_c * sigmoidf_(raw_w[i][e] + a.w0[c]));
                     }
-                    rs[tt * DKP + i] = r; ks[tt * DKP + i] = kk[e];
-                    us[tt * DKP + i] = u; aus[tt * DKP + i] = au; ws[tt * DKP + i] = w;
+                    rs[tt * DKP + idx] = raw_r[i][e]; ks[tt * DKP + idx] = raw_k[i][e];
+                    us[tt * DKP + idx] = u; aus[tt * DKP + idx] = au; ws[tt * DKP + idx] = w;
                 }
             } else {
-                for (int i = lane; i < DKP; i += 64) {
-                    float r = 0.f, k = 0.f;
-                    if (i < dk) {
-                        r = ld_f32(rp + t * a.r_stride + h * dk + i);
-                        k = ld_f32(kp + t * a.k_stride + h * dk + i);
-                        if (a.silu_in) { r = siluf_(r); k = siluf_(k); }
-                    }
-                    rs[tt * DKP + i] = r; ks[tt * DKP + i] = k;
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) {
+                    const int idx = e * 64 + lane;
+                    if (idx >= DKP) continue;
+                    float r = raw_r[i][e], k = raw_k[i][e];
+                    if (a.silu_in && idx < dk) { r = siluf_(r); k = siluf_(k); }
+                    rs[tt * DKP + idx] = r; ks[tt * DKP + idx] = k;
                 }
             }
         }
-        for (int e = tid; e < nc * CPB; e += NW * 64) {
-            const int tt = e / CPB, c = e - tt * CPB, jj = blockIdx.x * CPB + c;
-            float v = 0.f;
-            if (jj < dv) {
-                v = ld_f32(vp + (size_t)(t_lo + c0 + tt) * a.v_stride + h * dv + jj);
-                if (!DELTA && a.silu_in) v = siluf_(v);
-            }
-            vs[e] = v;
+#pragma unroll
+        for (int e = 0; e < SC_CH; ++e) {
+            const int x = e * (NW * 64) + tid;
+            if (x < nc * CPB) vs[x] = (!DELTA && a.silu_in) ? siluf_(raw_v[e]) : raw_v[e];
         }
+    };
+
+    ask(0);
+    for (int c0 = 0, turn = 0; c0 < n; c0 += SC_CH, turn ^= 1) {
+        const int nc = min(SC_CH, n - c0);
+        float* buf = lds + turn * BUF;
+        // the other buffer may still be walked by a slower wave; this one was last walked two
+        // stretches ago, before the barrier of the last stretch
+        stage(buf, nc);
+        if (c0 + SC_CH < n) ask(c0 + SC_CH);
         __syncthreads();
+        const float* rs = buf;
+        const float* ks = rs + SC_CH * DKP;
+        const float* us = ks + SC_CH * DKP;
+        const float* aus = us + SC_CH * DKP;
+        const float* ws = aus + SC_CH * DKP;
+        const float* vs = buf + NA * SC_CH * DKP;
         for (int tt = 0; tt < nc; ++tt) {
             const float vv = vs[tt * CPB + jc];
-            const int base = tt * DKP + pl * SC_R;
+            const int base = tt * DKP + pl * R;
             if (DELTA) {
                 float dot = 0.f;
 #pragma unroll
-                for (int ii = 0; ii < SC_R; ii += 4) {
+                for (int ii = 0; ii < R; ii += 4) {
                     const float4 u4 = *reinterpret_cast<const float4*>(us + base + ii);
                     dot = fmaf(u4.x, S[ii], dot); dot = fmaf(u4.y, S[ii + 1], dot);
                     dot = fmaf(u4.z, S[ii + 2], dot); dot = fmaf(u4.w, S[ii + 3], dot);
                 }
-                for (int o = CW; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
+                dot = group_sum(dot, P);
 #pragma unroll
-                for (int ii = 0; ii < SC_R; ii += 4) {
+                for (int ii = 0; ii < R; ii += 4) {
                     const float4 w4 = *reinterpret_cast<const float4*>(ws + base + ii);
                     const float4 a4 = *reinterpret_cast<const float4*>(aus + base + ii);
                     const float4 k4 = *reinterpret_cast<const float4*>(ks + base + ii);
@@ -147,7 +203,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                 }
             } else {
 #pragma unroll
-                for (int ii = 0; ii < SC_R; ii += 4) {
+                for (int ii = 0; ii < R; ii += 4) {
                     const float4 k4 = *reinterpret_cast<const float4*>(ks + base + ii);
                     S[ii] = fmaf(dec, S[ii], k4.x * vv); S[ii + 1] = fmaf(dec, S[ii + 1], k4.y * vv);
                     S[ii + 2] = fmaf(dec, S[ii + 2], k4.z * vv); S[ii + 3] = fmaf(dec, S[ii + 3], k4.w * vv);
@@ -155,34 +211,46 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
             }
             float o = 0.f;
 #pragma unroll
-            for (int ii = 0; ii < SC_R; ii += 4) {
+            for (int ii = 0; ii < R; ii += 4) {
                 const float4 r4 = *reinterpret_cast<const float4*>(rs + base + ii);
                 o = fmaf(r4.x, S[ii], o); o = fmaf(r4.y, S[ii + 1], o);
                 o = fmaf(r4.z, S[ii + 2], o); o = fmaf(r4.w, S[ii + 3], o);
             }
-            for (int s = CW; s < 64; s <<= 1) o += __shfl_xor(o, s, 64);
+            o = group_sum(o, P);
             if (pl == 0 && col_ok) a.out[(size_t)(t_lo + c0 + tt) * a.out_stride + h * dv + j] = o;
         }
     }
 #pragma unroll
-    for (int ii = 0; ii < SC_R; ++ii) {
-        const int i = pl * SC_R + ii;
+    for (int ii = 0; ii < R; ++ii) {
+        const int i = pl * R + ii;
         if (col_ok && i < dk) Sg[(size_t)i * dv + j] = S[ii];
     }
 }
 
-template <typename T, bool DELTA>
+template <typename T, bool DELTA, int R>
 int launch_scan(const ScanArgs& a, int num_rows, hipStream_t stream) {
-    const int P = a.P, DKP = P * SC_R;
+    const int P = a.P, DKP = P * R;
     // four waves a block unless that leaves most of the chip without a block
     const int cols4 = 4 * (64 / P);
     const long blocks4 = (long)((a.dv + cols4 - 1) / cols4) * a.H * num_rows;
     const int NW = blocks4 >= 256 ? 4 : 1;
     const int CPB = NW * (64 / P);
-    const size_t lds = sizeof(float) * ((DELTA ? 5 : 2) * SC_CH * DKP + SC_CH * CPB);
+    const size_t lds = sizeof(float) * 2 * ((DELTA ? 5 : 2) * SC_CH * DKP + SC_CH * CPB);
     dim3 grid((a.dv + CPB - 1) / CPB, a.H, num_rows);
-    if (NW == 4) linear_scan_kernel<T, DELTA, 4><<<grid, 256, lds, stream>>>(a);
-    else linear_scan_kernel<T, DELTA, 1><<<grid, 64, lds, stream>>>(a);
+    auto k4 = linear_scan_kernel<T, DELTA, R, 4>;
+    auto k1 = linear_scan_kernel<T, DELTA, R, 1>;
+    if (lds > 64 * 1024) {
+        // more LDS than a kernel gets unasked (the delta form with more than 128 key rows)
+        static bool asked[2] = {};
+        if (!asked[NW == 4]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(NW == 4 ? k4 : k1),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            RI_REQUIRE(e == hipSuccess, "ri_linear_scan: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+            asked[NW == 4] = true;
+        }
+    }
+    if (NW == 4) k4<<<grid, 256, lds, stream>>>(a);
+    else k1<<<grid, 64, lds, stream>>>(a);
     return 0;
 }
 
@@ -208,17 +276,23 @@ extern "C" int ri_linear_scan(
     RI_REQUIRE(H <= 65535 && num_rows <= 65535, "ri_linear_scan: too many heads or rows for the grid");
     if (delta) RI_REQUIRE(wl && al && w0 && ab && wl_stride >= H * dk && al_stride >= H * dk, "ri_linear_scan: the delta form needs wl, al, w0, ab");
     else RI_REQUIRE(decay, "ri_linear_scan: the decay form needs a decay for each head");
+    // key rows a thread: 8, or 16 where 8 would need more than the 16 lanes a column may have
+    const int R = dk <= 128 ? 8 : 16;
     int P = 1;
-    while (P * SC_R < dk) P *= 2;
+    while (P * R < dk) P *= 2;
     ScanArgs a;
     a.r = r; a.k = k; a.v = v; a.wl = wl; a.al = al;
     a.r_stride = r_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.wl_stride = wl_stride; a.al_stride = al_stride;
     a.w0 = w0; a.ab = ab; a.decay = decay; a.state = state; a.out = out; a.out_stride = out_stride;
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = silu_in; a.unit_eps = unit_eps; a.decay_c = decay_c;
-    if (dtype == RI_F32) { if (delta) launch_scan<float, true>(a, num_rows, stream); else launch_scan<float, false>(a, num_rows, stream); }
-    else if (dtype == RI_BF16) { if (delta) launch_scan<bf16_t, true>(a, num_rows, stream); else launch_scan<bf16_t, false>(a, num_rows, stream); }
+    int rc;
+#define RI_SCAN(TT, DD) (R == 8 ? launch_scan<TT, DD, 8>(a, num_rows, stream) : launch_scan<TT, DD, 16>(a, num_rows, stream))
+    if (dtype == RI_F32) rc = delta ? RI_SCAN(float, true) : RI_SCAN(float, false);
+    else if (dtype == RI_BF16) rc = delta ? RI_SCAN(bf16_t, true) : RI_SCAN(bf16_t, false);
     else return ri_fail("ri_linear_scan: unknown dtype %d", dtype);
+#undef RI_SCAN
+    if (rc) return rc;
     RI_LAUNCHED("ri_linear_scan");
     return 0;
 }

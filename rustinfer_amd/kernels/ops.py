@@ -929,10 +929,19 @@ def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: i
     _i32(ctx.q_start, "q_start", ctx.num_rows)
     _i32(ctx.kv_lens, "kv_lens", ctx.num_rows)
     vcos, vsin, vrows = _rot_tables(value_rotary, dv, "window_attention (values)")
-    _check(_lib().ri_attention_window(
+    lib = _lib()
+    # a step of single tokens divides each row's keys between blocks, through a workspace
+    single, ws, need = int(ctx.max_q_len == 1 and T <= ctx.num_rows), None, 0
+    if single:
+        lib.ri_attention_window_workspace.restype = ctypes.c_size_t
+        need = lib.ri_attention_window_workspace(T, H, dk, dv, int(window), int(ctx.max_kv_len))
+        if need:
+            ws = ctx.workspace.get("attn.window_partials", need, 1, torch.float32)
+    _check(lib.ri_attention_window(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
         H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
-        ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _stream()))
+        ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)),
+        single, int(ctx.max_kv_len), _ptr(ws), ctypes.c_size_t(need), _stream()))
 
 
 # ---------------------------------------------------------------------------
