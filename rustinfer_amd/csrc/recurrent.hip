@@ -19,15 +19,14 @@
 // thread.  The vectors of a stretch of eight tokens are asked for a stretch ahead, brought into one
 // of two LDS buffers already activated, and read by the walk as broadcasts.  What a token adds up, and in which order, does not depend on how the request was
 // cut into steps, so the state and the outputs have the same bits for every cut.
-// A block holds NW waves (64 NW / P columns); with few (request, head) pairs a wave a block, so
-// that the chip has blocks enough.
+// A block holds four waves (256 / P columns) that share the staging, or one wave for a head of
+// no more than 64 threads.
 #include "common.h"
 #include <math.h>
 
 namespace {
 
 constexpr int SC_CH = 8;         // tokens a stretch
-constexpr int SC_EPL = 4;        // most key rows a lane stages for one token (64 lanes x 4 >= 256)
 
 struct ScanArgs {
     const void *r, *k, *v, *wl, *al;
@@ -41,8 +40,11 @@ struct ScanArgs {
     float unit_eps, decay_c;
 };
 
-__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
-__device__ __forceinline__ float siluf_(float z) { return z / (1.f + expf(-z)); }
+// exp on the hardware's 2^x (an error of a unit or two in the last place of 32 bits) and a division
+// without the library's special cases: the staging of a stretch is a third of the walk's time
+__device__ __forceinline__ float expf_(float z) { return __expf(z); }
+__device__ __forceinline__ float sigmoidf_(float z) { return __fdividef(1.f, 1.f + __expf(-z)); }
+__device__ __forceinline__ float siluf_(float z) { return __fdividef(z, 1.f + __expf(-z)); }
 
 // Sum over the P adjacent lanes that share a column (P a power of two up to 16), every lane
 // getting the same bits: exchanges inside a quad, between the quads of half a row, between the
@@ -59,8 +61,20 @@ __device__ __forceinline__ float group_sum(float x, int P) {
     return x;
 }
 
-template <typename T, bool DELTA, int R, int NW>
+// EPL: key rows a lane stages for one token (64 EPL >= dk)
+// Sum over the 64 lanes with exchanges that stay in the vector unit, then one read of each row
+// of 16 lanes; the same bits in every lane.
+__device__ __forceinline__ float wave_sum_rows(float x) {
+    x = group_sum(x, 16);
+    return ((__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 0))
+           + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 16)))
+          + (__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 32))
+           + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 48))));
+}
+
+template <typename T, bool DELTA, int R, int NW, int EPL>
 __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) {
+    constexpr int SC_EPL = EPL;
     extern __shared__ __align__(16) float lds[];
     constexpr int TPW = SC_CH / NW;                    // tokens of a stretch a wave stages
     constexpr int NA = DELTA ? 5 : 2;
@@ -110,6 +124,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         }
 #pragma unroll
         for (int e = 0; e < SC_CH; ++e) {
+            if (e * (NW * 64) >= SC_CH * CPB) break;    // a stretch has SC_CH * CPB values: SC_CH / P a thread
             const int x = e * (NW * 64) + tid;
             const int tt = x / CPB, c = x - tt * CPB, jj = blockIdx.x * CPB + c;
             raw_v[e] = (x < nc * CPB && jj < dv) ? ld_f32(vp + (size_t)(t_lo + c0 + tt) * a.v_stride + h * dv + jj) : 0.f;
@@ -130,7 +145,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                 float ssq = 0.f;
 #pragma unroll
                 for (int e = 0; e < SC_EPL; ++e) ssq = fmaf(raw_k[i][e], raw_k[i][e], ssq);
-                ssq = wave_sum(ssq);
+                ssq = wave_sum_rows(ssq);
                 const float inv = 1.f / sqrtf(ssq + a.unit_eps);
 #pragma unroll
                 for (int e = 0; e < SC_EPL; ++e) {
@@ -141,7 +156,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                         const int c = h * dk + idx;
                         u = raw_k[i][e] * inv;
                         au = sigmoidf_(raw_a[i][e] + a.ab[c]) * u;
-                        w = expf(-a.decay_c * sigmoidf_(raw_w[i][e] + a.w0[c]));
+                        w = expf_(-a.decay_c * sigmoidf_(raw_w[i][e] + a.w0[c]));
                     }
                     rs[tt * DKP + idx] = raw_r[i][e]; ks[tt * DKP + idx] = raw_k[i][e];
                     us[tt * DKP + idx] = u; aus[tt * DKP + idx] = au; ws[tt * DKP + idx] = w;
@@ -159,6 +174,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         }
 #pragma unroll
         for (int e = 0; e < SC_CH; ++e) {
+            if (e * (NW * 64) >= SC_CH * CPB) break;
             const int x = e * (NW * 64) + tid;
             if (x < nc * CPB) vs[x] = (!DELTA && a.silu_in) ? siluf_(raw_v[e]) : raw_v[e];
         }
@@ -227,31 +243,39 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
     }
 }
 
-template <typename T, bool DELTA, int R>
-int launch_scan(const ScanArgs& a, int num_rows, hipStream_t stream) {
-    const int P = a.P, DKP = P * R;
-    // four waves a block unless that leaves most of the chip without a block
-    const int cols4 = 4 * (64 / P);
-    const long blocks4 = (long)((a.dv + cols4 - 1) / cols4) * a.H * num_rows;
-    const int NW = blocks4 >= 256 ? 4 : 1;
-    const int CPB = NW * (64 / P);
+template <typename T, bool DELTA, int R, int NW, int EPL>
+int launch_scan_as(const ScanArgs& a, int num_rows, hipStream_t stream) {
+    const int P = a.P, DKP = P * R, CPB = NW * (64 / P);
     const size_t lds = sizeof(float) * 2 * ((DELTA ? 5 : 2) * SC_CH * DKP + SC_CH * CPB);
     dim3 grid((a.dv + CPB - 1) / CPB, a.H, num_rows);
-    auto k4 = linear_scan_kernel<T, DELTA, R, 4>;
-    auto k1 = linear_scan_kernel<T, DELTA, R, 1>;
+    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL>;
     if (lds > 64 * 1024) {
         // more LDS than a kernel gets unasked (the delta form with more than 128 key rows)
-        static bool asked[2] = {};
-        if (!asked[NW == 4]) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(NW == 4 ? k4 : k1),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        static bool asked = false;
+        if (!asked) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
             RI_REQUIRE(e == hipSuccess, "ri_linear_scan: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-            asked[NW == 4] = true;
+            asked = true;
         }
     }
-    if (NW == 4) k4<<<grid, 256, lds, stream>>>(a);
-    else k1<<<grid, 64, lds, stream>>>(a);
+    kernel<<<grid, NW * 64, lds, stream>>>(a);
     return 0;
+}
+
+template <typename T, bool DELTA, int R>
+int launch_scan(const ScanArgs& a, int num_rows, hipStream_t stream) {
+    // Four waves a block share the staging of a stretch (a wave alone spends more instructions on
+    // staging than on the walk); one wave where a head has no more than 64 threads.
+    const bool four = (long)a.dv * a.P > 64;
+    const int epl = (a.dk + 63) / 64;
+    if (four) {
+        if (epl == 1) return launch_scan_as<T, DELTA, R, 4, 1>(a, num_rows, stream);
+        if (epl == 2) return launch_scan_as<T, DELTA, R, 4, 2>(a, num_rows, stream);
+        return launch_scan_as<T, DELTA, R, 4, 4>(a, num_rows, stream);
+    }
+    if (epl == 1) return launch_scan_as<T, DELTA, R, 1, 1>(a, num_rows, stream);
+    if (epl == 2) return launch_scan_as<T, DELTA, R, 1, 2>(a, num_rows, stream);
+    return launch_scan_as<T, DELTA, R, 1, 4>(a, num_rows, stream);
 }
 
 }  // namespace
