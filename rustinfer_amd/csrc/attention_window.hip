@@ -148,15 +148,19 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 
     const int tile = blockIdx.x, g = blockIdx.y, G = H / Hkv;
     int b = -1, t0 = 0, nt = 0, before = 0;
-    for (int r = 0; r < num_rows; ++r) {
-        const int lo = cu_q[r], ql = cu_q[r + 1] - lo, tiles = (ql + TQ - 1) / TQ;
-        if (tile < before + tiles) {
-            b = r;
-            t0 = lo + (tile - before) * TQ;
-            nt = min(TQ, lo + ql - t0);
-            break;
+    if (slots > 0) {                                   // a tile a row: row `tile` and its one token, if it has one
+        if (tile < num_rows && cu_q[tile + 1] - cu_q[tile] > 0) { b = tile; t0 = cu_q[tile]; nt = 1; }
+    } else {
+        for (int r = 0; r < num_rows; ++r) {
+            const int lo = cu_q[r], ql = cu_q[r + 1] - lo, tiles = (ql + TQ - 1) / TQ;
+            if (tile < before + tiles) {
+                b = r;
+                t0 = lo + (tile - before) * TQ;
+                nt = min(TQ, lo + ql - t0);
+                break;
+            }
+            before += tiles;
         }
-        before += tiles;
     }
     if (b < 0) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -259,6 +263,8 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi) {
             if (bi >= batches) break;
+            // rows of this batch that exist for this wave (a step of single tokens has G rows a tile)
+            const int nrb = min(4, (R - wave + 3) / 4 - 4 * bi);
             float s[4] = {0.f, 0.f, 0.f, 0.f};
             const float* kr = Ks + (lane < NK ? lane : 0) * ks_stride;
 #pragma unroll 2
@@ -266,6 +272,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
                 const float4 k4 = *reinterpret_cast<const float4*>(kr + dd);
 #pragma unroll
                 for (int rb = 0; rb < 4; ++rb) {
+                    if (rb >= nrb) break;
                     const float4 q4 = *reinterpret_cast<const float4*>(Qs + (wave + 4 * (4 * bi + rb)) * dkp + dd);
                     s[rb] = fmaf(q4.x, k4.x, s[rb]);
                     s[rb] = fmaf(q4.y, k4.y, s[rb]);
@@ -286,6 +293,8 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi) {
             if (bi >= batches) break;
+            const int nrb = min(4, (R - wave + 3) / 4 - 4 * bi);
+            if (nrb <= 0) break;
 #pragma unroll 1
             for (int jj = 0; jj < NK; jj += 4) {
                 float4 p4[4];
@@ -300,6 +309,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
                         const float v = d < dv ? Vs[(jj + u) * vs_stride + d] : 0.f;
 #pragma unroll
                         for (int rb = 0; rb < 4; ++rb) {
+                            if (rb >= nrb) break;
                             const float pv = u == 0 ? p4[rb].x : u == 1 ? p4[rb].y : u == 2 ? p4[rb].z : p4[rb].w;
                             acc_b[4 * bi + rb][c] = fmaf(pv, v, acc_b[4 * bi + rb][c]);
                         }
@@ -556,5 +566,313 @@ extern "C" int ri_attention_window(
         return ri_fail("ri_attention_window: unknown dtype %d", dtype);
     if (rc) return rc;
     RI_LAUNCHED("ri_attention_window");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Prompt portions on the matrix cores, in 32-bit: v_mfma_f32_32x32x2_f32 for both products, so
+// that scores, softmax weights and weighted sums keep 32 bits (the bfloat16 matrix instructions
+// would round the weights).  A wave owns 32 query tokens of one head and computes, for a tile of
+// 32 keys, S^T = K Q^T (keys down the registers, ONE query a lane: the softmax of a query is a
+// reduction over the lane's own 16 registers and one exchange with the lane 32 further on), then
+// O^T += V^T P^T with the weights used where they lie: step i of the second product takes key
+// 8 (i / 4) + i % 4 of the tile from the lower 32 lanes and key 8 (i / 4) + 4 + i % 4 from the
+// upper, which is what accumulator register i of the first product holds.  The query's features
+// stay in registers for the whole tile; keys and values of 64 positions at a time go through LDS
+// as 32-bit for the four waves of a block: the heads of one key/value head (four at a time), or,
+// for fewer than four heads a key/value head, consecutive tiles of 32 tokens.  Key tiles are
+// aligned to absolute positions and a query's arithmetic does not depend on its place in the tile:
+// a token's output has the same bits however its request was cut.
+// QU: 8-feature units of the (zero-padded) key head; FT: 32-feature tiles of the value head.
+// ---------------------------------------------------------------------------
+namespace {
+
+typedef float aw_f16 __attribute__((ext_vector_type(16)));
+constexpr int AM_KEYS = 64;      // keys a stage
+
+size_t am_lds_bytes(int QU, int dv) {
+    const size_t stage = (size_t)AM_KEYS * (8 * QU + 4) + (size_t)AM_KEYS * (dv + 8);
+    const size_t outs = (size_t)128 * dv;
+    return sizeof(float) * (64 + (stage > outs ? stage : outs));
+}
+
+template <typename T, int QU, int FT>
+__global__ __launch_bounds__(256) void attn_window_mfma_kernel(
+        const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
+        const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
+        const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
+        int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window,
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+    extern __shared__ __align__(16) float lds[];
+    constexpr int DKP = 8 * QU, KS = DKP + 4;
+    const int vs_stride = dv + 8;
+    int* koff = reinterpret_cast<int*>(lds);           // [64]
+    float* Ks = lds + 64;                              // [64][DKP + 4]
+    float* Vs = Ks + AM_KEYS * KS;                     // [64][dv + 8]
+    float* Os = Ks;                                    // [4 waves][32][dv], after the last stage
+
+    const int G = H / Hkv, HB = G < 4 ? G : 4, SB = 4 / HB, TQB = 32 * SB;
+    const int g = blockIdx.y, hgroup = blockIdx.z;
+    int b = -1, t0 = 0, nt = 0, before = 0;
+    for (int r = 0; r < num_rows; ++r) {
+        const int lo = cu_q[r], ql = cu_q[r + 1] - lo, tiles = (ql + TQB - 1) / TQB;
+        if ((int)blockIdx.x < before + tiles) {
+            b = r;
+            t0 = lo + ((int)blockIdx.x - before) * TQB;
+            nt = min(TQB, lo + ql - t0);
+            break;
+        }
+        before += tiles;
+    }
+    if (b < 0) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 31, lh = lane >> 5;          // the lane's query, and which half of the key pairs
+    const int p0 = q_start[b] + (t0 - cu_q[b]);
+    const int kv_len = kv_lens[b];
+    const int blk_last = min(kv_len, p0 + nt);
+    const int blk_first = window > 0 ? max(0, p0 + 1 - window) : 0;
+    // this wave's 32 tokens and head
+    const int sub = wave / HB, hh = hgroup * 4 + wave % HB;
+    const bool wave_on = sub < SB && hh < G && nt - 32 * sub > 0;
+    const int t0w = t0 + 32 * sub, ntw = wave_on ? min(32, nt - 32 * sub) : 0, p0w = p0 + 32 * sub;
+    const int head = g * G + (hh < G ? hh : 0);
+    const int w_last = wave_on ? min(kv_len, p0w + ntw) : 0;
+    const int w_first = window > 0 ? max(0, p0w + 1 - window) : 0;
+    const bool row_on = lq < ntw;
+    const int pq = p0w + lq;                           // the lane's query position
+
+    // the query's features, in the order the products take them: unit u, step c -> feature 8 u + 4 lh + c
+    float qr[QU * 4];
+#pragma unroll
+    for (int u = 0; u < QU; ++u)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int d = 8 * u + 4 * lh + c;
+            qr[u * 4 + c] = (row_on && d < dk) ? ld_f32(q + (size_t)(t0w + lq) * q_stride + head * dk + d) * scale : 0.f;
+        }
+    // the padding of the key rows beyond dk stays zero: the staging writes features below dk only
+    for (int e = tid; e < AM_KEYS * KS; e += 256) Ks[e] = 0.f;
+
+    aw_f16 o[FT];
+#pragma unroll
+    for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[ft][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    for (int st = blk_first / AM_KEYS; st * AM_KEYS < blk_last; ++st) {
+        const int j_base = st * AM_KEYS;
+        __syncthreads();                               // the last stage has been used (first pass: the zeros are written)
+        if (tid < AM_KEYS) {
+            const int j = j_base + tid;
+            int off = -1;
+            if (j < blk_last && j >= blk_first) {
+                const int pid = table[(size_t)b * max_blocks + j / page];
+                if (pid >= 0) off = (pid * Hkv + g) * page + j % page;
+            }
+            koff[tid] = off;
+        }
+        __syncthreads();
+        constexpr int VL = 16 / sizeof(T);
+        if (dk % VL == 0) {
+            const int pieces = dk / VL;
+            for (int e = tid; e < AM_KEYS * pieces; e += 256) {
+                const int jj = e / pieces, pc = e - jj * pieces, off = koff[jj];
+                float f[VL];
+#pragma unroll
+                for (int u = 0; u < VL; ++u) f[u] = 0.f;
+                if (off >= 0) ld_vec16(kc + (size_t)off * dk + pc * VL, f);
+#pragma unroll
+                for (int u = 0; u < VL; u += 4)
+                    *reinterpret_cast<float4*>(Ks + jj * KS + pc * VL + u) = make_float4(f[u], f[u + 1], f[u + 2], f[u + 3]);
+            }
+        } else {
+            for (int e = tid; e < AM_KEYS * dk; e += 256) {
+                const int jj = e / dk, dd = e - jj * dk, off = koff[jj];
+                Ks[jj * KS + dd] = off >= 0 ? ld_f32(kc + (size_t)off * dk + dd) : 0.f;
+            }
+        }
+        if (page % VL == 0) {
+            const int runs = AM_KEYS / VL;
+            for (int e = tid; e < runs * dv; e += 256) {
+                const int d = e / runs, jj0 = (e - d * runs) * VL;
+                float f[VL];
+#pragma unroll
+                for (int u = 0; u < VL; ++u) f[u] = 0.f;
+                int first = -1;
+#pragma unroll
+                for (int u = 0; u < VL; ++u) if (first < 0 && koff[jj0 + u] >= 0) first = u;
+                if (first >= 0) {
+                    const int off = koff[jj0 + first] - first;
+                    ld_vec16(vc + (size_t)(off / page) * page * dv + (size_t)d * page + off % page, f);
+                }
+#pragma unroll
+                for (int u = 0; u < VL; ++u) Vs[(jj0 + u) * vs_stride + d] = koff[jj0 + u] >= 0 ? f[u] : 0.f;
+            }
+        } else {
+            const int jj = tid & 63, off = koff[jj];
+            const size_t vbase = off >= 0 ? (size_t)(off / page) * page * dv + off % page : 0;
+            for (int d = tid >> 6; d < dv; d += 4)
+                Vs[jj * vs_stride + d] = off >= 0 ? ld_f32(vc + vbase + (size_t)d * page) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 1
+        for (int half = 0; half < 2; ++half) {
+            const int kt0 = j_base + 32 * half;        // first key of the tile
+            if (kt0 >= w_last || kt0 + 32 <= w_first) continue;     // none of the wave's queries sees it (the same for all lanes)
+            // S^T = K Q^T (the scale is in the query)
+            aw_f16 s;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[i] = 0.f;
+            const float* krow = Ks + (32 * half + lq) * KS + 4 * lh;
+#pragma unroll
+            for (int u = 0; u < QU; ++u) {
+                const float4 k4 = *reinterpret_cast<const float4*>(krow + 8 * u);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.x, qr[u * 4 + 0], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.y, qr[u * 4 + 1], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.z, qr[u * 4 + 2], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.w, qr[u * 4 + 3], s, 0, 0, 0);
+            }
+            // register i: key kt0 + 8 (i / 4) + 4 lh + i % 4, for the lane's query
+            const int j_lo = window > 0 ? pq + 1 - window : 0, j_hi = min(pq + 1, kv_len);
+            float mt = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int j = kt0 + 8 * (i >> 2) + 4 * lh + (i & 3);
+                const bool vis = row_on && j >= j_lo && j < j_hi;
+                s[i] = vis ? s[i] : -INFINITY;
+                mt = fmaxf(mt, s[i]);
+            }
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m, mt);
+            const bool any = m_new > -INFINITY;        // else the query has seen no key yet: nothing to add
+            const float alpha = any ? expf(m - m_new) : 1.f;
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[i] = (any && s[i] > -INFINITY) ? expf(s[i] - m_new) : 0.f;
+                psum += s[i];
+            }
+            l = l * alpha + psum;
+            m = m_new;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[ft][i] *= alpha;
+            // O^T += V^T P^T
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const int f = 32 * ft + lq;
+                if (32 * ft >= dv) continue;
+                const float* vcol = Vs + (32 * half + 4 * lh) * vs_stride + (f < dv ? f : 0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float a = f < dv ? vcol[(8 * (i >> 2) + (i & 3)) * vs_stride] : 0.f;
+                    o[ft] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[i], o[ft], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // the sums of a query lie in the lane of its lower and of its upper half: add the two l
+    l += __shfl_xor(l, 32, 64);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    __syncthreads();                                   // the last keys and values have been used
+    float* ow = Os + (size_t)wave * 32 * dv;
+    if (wave_on) {
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int f = 32 * ft + 8 * (i >> 2) + 4 * lh + (i & 3);
+                if (f < dv) ow[lq * dv + f] = o[ft][i] * inv;
+            }
+    }
+    __syncthreads();
+    if (!wave_on) return;
+    const int vh = dv >> 1;
+    for (int r = 0; r < ntw; ++r) {
+        T* orow = out + (size_t)(t0w + r) * out_stride + head * dv;
+        if (vcos == nullptr) {
+            for (int f = lane; f < dv; f += 64) st_f32(orow + f, ow[r * dv + f]);
+        } else {
+            const int p = p0w + r;
+            for (int mm = lane; mm < vh; mm += 64) {
+                const int i0 = v_interleaved ? 2 * mm : mm, i1 = v_interleaved ? 2 * mm + 1 : mm + vh;
+                const float a = ow[r * dv + i0], bb = ow[r * dv + i1];
+                const float c = vcos[(size_t)p * vh + mm], s_ = vsin[(size_t)p * vh + mm];
+                st_f32(orow + i0, a * c + bb * s_);
+                st_f32(orow + i1, bb * c - a * s_);
+            }
+        }
+    }
+}
+
+template <typename T, int QU, int FT>
+int am_launch_as(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
+                 const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
+                 int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, hipStream_t stream) {
+    const int G = H / Hkv, HB = G < 4 ? G : 4, SB = 4 / HB, TQB = 32 * SB;
+    const size_t lds = am_lds_bytes(QU, dv);
+    auto kernel = attn_window_mfma_kernel<T, QU, FT>;
+    if (lds > 64 * 1024) {
+        static bool asked = false;
+        if (!asked) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            RI_REQUIRE(e == hipSuccess, "ri_attention_window: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+            asked = true;
+        }
+    }
+    const int tiles = (Tn + TQB - 1) / TQB + num_rows;
+    kernel<<<dim3(tiles, Hkv, (G + 3) / 4), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start,
+                                                               kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved);
+    return 0;
+}
+
+template <typename T>
+int am_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
+              const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
+              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, hipStream_t stream) {
+#define RI_AM(QU, FT) return am_launch_as<T, QU, FT>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, \
+        num_rows, Tn, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream)
+    if (dk <= 64) { if (dv <= 64) RI_AM(8, 2); if (dv <= 128) RI_AM(8, 4); RI_AM(8, 8); }
+    if (dk <= 128) { if (dv <= 64) RI_AM(16, 2); if (dv <= 128) RI_AM(16, 4); RI_AM(16, 8); }
+    if (dv <= 64) RI_AM(32, 2);
+    if (dv <= 128) RI_AM(32, 4);
+    RI_AM(32, 8);
+#undef RI_AM
+}
+
+}  // namespace
+
+extern "C" int ri_attention_window_mfma_supported(int H, int Hkv, int dk, int dv) {
+    if (!ri_attention_window_supported(H, Hkv, dk, dv)) return 0;
+    const int QU = dk <= 64 ? 8 : dk <= 128 ? 16 : 32;
+    return am_lds_bytes(QU, dv) <= 160 * 1024;
+}
+
+// The same attention as ri_attention_window for steps with prompt portions, on the 32-bit matrix
+// instructions.
+extern "C" int ri_attention_window_mfma(
+        const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kc, const void* vc,
+        int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
+        const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
+        float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
+        hipStream_t stream) {
+    RI_REQUIRE(ri_attention_window_mfma_supported(H, Hkv, dk, dv), "ri_attention_window_mfma: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
+    RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window_mfma: bad sizes");
+    RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window_mfma: row strides too small");
+    if (vcos) RI_REQUIRE(vsin && dv % 2 == 0 && v_table_rows > 0, "ri_attention_window_mfma: a turned value needs an even size and both tables");
+    if (T == 0 || num_rows == 0) return 0;
+    RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_window_mfma: null pointer");
+    RI_REQUIRE(Hkv <= 65535, "ri_attention_window_mfma: too many key/value heads for the grid");
+    int rc;
+    if (dtype == RI_F32)
+        rc = am_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+    else if (dtype == RI_BF16)
+        rc = am_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+    else
+        return ri_fail("ri_attention_window_mfma: unknown dtype %d", dtype);
+    if (rc) return rc;
+    RI_LAUNCHED("ri_attention_window_mfma");
     return 0;
 }

@@ -61,6 +61,14 @@ __device__ __forceinline__ float group_sum(float x, int P) {
     return x;
 }
 
+// The block's barrier for data that passes through LDS only: the wave's LDS writes are done, then
+// the barrier.  __syncthreads() would also wait for the global loads just asked for and for the
+// outputs just stored, a trip to memory for every stretch of eight tokens (it was two thirds of
+// the walk's time).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // EPL: key rows a lane stages for one token (64 EPL >= dk)
 // Sum over the 64 lanes with exchanges that stay in the vector unit, then one read of each row
 // of 16 lanes; the same bits in every lane.
@@ -188,13 +196,14 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         // stretches ago, before the barrier of the last stretch
         stage(buf, nc);
         if (c0 + SC_CH < n) ask(c0 + SC_CH);
-        __syncthreads();
+        lds_barrier();
         const float* rs = buf;
         const float* ks = rs + SC_CH * DKP;
         const float* us = ks + SC_CH * DKP;
         const float* aus = us + SC_CH * DKP;
         const float* ws = aus + SC_CH * DKP;
         const float* vs = buf + NA * SC_CH * DKP;
+#pragma unroll 4
         for (int tt = 0; tt < nc; ++tt) {
             const float vv = vs[tt * CPB + jc];
             const int base = tt * DKP + pl * R;

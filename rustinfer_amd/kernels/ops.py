@@ -903,6 +903,9 @@ def rotate_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torc
         int(bool(write_kv)), _stream()))
 
 
+WINDOW_ATTENTION_MFMA = True     # steps with prompt portions take the matrix-instruction kernel (False: the FMA one, for comparison)
+
+
 def window_attention_supported(H: int, Hkv: int, dk: int, dv: int) -> bool:
     return bool(_lib().ri_attention_window_supported(H, Hkv, dk, dv))
 
@@ -930,6 +933,13 @@ def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: i
     _i32(ctx.kv_lens, "kv_lens", ctx.num_rows)
     vcos, vsin, vrows = _rot_tables(value_rotary, dv, "window_attention (values)")
     lib = _lib()
+    if ctx.max_q_len > 1 and WINDOW_ATTENTION_MFMA and lib.ri_attention_window_mfma_supported(H, Hkv, dk, dv):
+        # steps with prompt portions: both products on the 32-bit matrix instructions
+        _check(lib.ri_attention_window_mfma(
+            _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
+            H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
+            ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _stream()))
+        return
     # a step of single tokens divides each row's keys between blocks, through a workspace
     single, ws, need = int(ctx.max_q_len == 1 and T <= ctx.num_rows), None, 0
     if single:

@@ -207,11 +207,20 @@ PART_TOL = {"float32": 2e-5, "bfloat16": 4e-2}
 CUTS = (13, 1, 1, 2, 30, 1, 7, 2, 1, 1, 1, 1, 40, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 5)
 
 
+@pytest.fixture(params=["matrix", "fma"])
+def portion_kernel(request):
+    """Steps with prompt portions on the matrix-instruction kernel (the default) and on the FMA one."""
+    from rustinfer_amd.kernels import ops
+    keep, ops.WINDOW_ATTENTION_MFMA = ops.WINDOW_ATTENTION_MFMA, request.param == "matrix"
+    yield request.param
+    ops.WINDOW_ATTENTION_MFMA = keep
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,G,dk,dv,rot,window,scale,inter", [
     (4, 2, 16, 24, 8, 9, 0.3, False), (3, 3, 40, 36, 40, 1, 0.2, False), (8, 1, 32, 16, 2, 33, 0.18, True),
     (2, 2, 128, 128, 64, 70, 0.09, False), (5, 5, 72, 200, 72, 17, 0.12, False), (6, 2, 64, 64, 64, 500, 0.125, False)])
-def test_window_attention_alone(dtype, H, G, dk, dv, rot, window, scale, inter):
+def test_window_attention_alone(dtype, H, G, dk, dv, rot, window, scale, inter, portion_kernel):
     from rustinfer_amd.parts import RotaryEmbedding, WindowAttention
     d = 48
     pe, vpe = RotaryEmbedding(dk, 300.0, rot_dim=rot), RotaryEmbedding(dv, 300.0)
@@ -301,7 +310,7 @@ def test_dense_feed_forward_and_capped_head(dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("decoded", [False, True])
-def test_one_key_decides_at_the_windows_edge(dtype, decoded):
+def test_one_key_decides_at_the_windows_edge(dtype, decoded, portion_kernel):
     """A query that matches one far key a hundredfold: with the key on the window's last
     position the output is that key's value (turned by the distance), one position further out
     it is not seen at all.  Among 300 keys, across pages, in a prompt and in single tokens."""
