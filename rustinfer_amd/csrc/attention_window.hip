@@ -15,6 +15,9 @@
 // rotate_kv_write: one block a token; rotates q in place over its first `rot` features (feature
 // i with i + rot/2), writes the rotated key and the turned value into the token's page.
 //
+// Three attention kernels: attn_window (FMA, any mix of rows; below), attn_window_mfma (steps with
+// prompt portions, on the 32-bit matrix instructions; further down) and attn_window_decode with
+// attn_window_combine (steps of single tokens, a row's keys divided between waves).
 // attn_window: a block of four waves owns up to 32 query rows: TQ = 32 / G consecutive tokens of
 // one request (G = H / Hkv query heads each) on one key/value head; a row of one token is a tile
 // of its own.  Keys go by in blocks of NK (64 where LDS allows) aligned to absolute positions, so
@@ -133,10 +136,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
         const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window, int TQ, int NK,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved,
-        int slots, float* __restrict__ part_ml, float* __restrict__ part_o) {
-    // slots > 0 (steps of single tokens): the block takes ONE block of keys, the blockIdx.z-th of
-    // its row's window, and leaves its partial result for attn_window_combine_kernel
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
     extern __shared__ __align__(16) float lds[];
     const int dkp = (dk + 3) & ~3, ks_stride = dkp + 4, vs_stride = dv + 1;
     float* Qs = lds;                                   // [AW_ROWS][dkp]
@@ -148,19 +148,15 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 
     const int tile = blockIdx.x, g = blockIdx.y, G = H / Hkv;
     int b = -1, t0 = 0, nt = 0, before = 0;
-    if (slots > 0) {                                   // a tile a row: row `tile` and its one token, if it has one
-        if (tile < num_rows && cu_q[tile + 1] - cu_q[tile] > 0) { b = tile; t0 = cu_q[tile]; nt = 1; }
-    } else {
-        for (int r = 0; r < num_rows; ++r) {
-            const int lo = cu_q[r], ql = cu_q[r + 1] - lo, tiles = (ql + TQ - 1) / TQ;
-            if (tile < before + tiles) {
-                b = r;
-                t0 = lo + (tile - before) * TQ;
-                nt = min(TQ, lo + ql - t0);
-                break;
-            }
-            before += tiles;
+    for (int r = 0; r < num_rows; ++r) {
+        const int lo = cu_q[r], ql = cu_q[r + 1] - lo, tiles = (ql + TQ - 1) / TQ;
+        if (tile < before + tiles) {
+            b = r;
+            t0 = lo + (tile - before) * TQ;
+            nt = min(TQ, lo + ql - t0);
+            break;
         }
+        before += tiles;
     }
     if (b < 0) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -188,13 +184,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
         row_lo[i] = window > 0 ? max(0, p + 1 - window) : 0;
     }
 
-    int kb_lo = first_key / NK, kb_hi = (last_visible + NK - 1) / NK;
-    if (slots > 0) {
-        kb_lo += blockIdx.z;
-        kb_hi = min(kb_hi, kb_lo + 1);
-        if (kb_lo >= kb_hi) return;                    // the row's window has fewer blocks of keys
-    }
-    for (int kb = kb_lo; kb < kb_hi; ++kb) {
+    for (int kb = first_key / NK; kb * NK < last_visible; ++kb) {
         const int j_base = kb * NK;
         __syncthreads();                               // the last block of keys has been used (first pass: Qs is written)
         if (tid < NK) {
@@ -320,21 +310,6 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) aw_merge<NC>(m[i], l[i], acc[i], m_b[i], l_b[i], acc_b[i]);
     }
-    if (slots > 0) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int r = wave + 4 * i;
-            if (r >= R) continue;
-            const size_t at = ((size_t)(t0 + r / G) * H + (g * G + r % G)) * slots + blockIdx.z;
-            if (lane == 0) { part_ml[at * 2] = m[i]; part_ml[at * 2 + 1] = l[i]; }
-#pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                const int d = lane + 64 * c;
-                if (d < dv) part_o[at * dv + d] = acc[i][c];
-            }
-        }
-        return;
-    }
     if (vcos == nullptr) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -378,8 +353,8 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 }
 
 // Steps of single tokens: merge the partial results of a row's blocks of keys in ascending order
-// (the order and the arithmetic of the loop in attn_window_kernel, so a token's output has the
-// same bits as there), divide, turn back, write.  One wave a (token, head).
+// (the order and the arithmetic of the loop in attn_window_kernel), divide, turn back, write.
+// One wave a (token, head).
 template <typename T, int NC>
 __global__ __launch_bounds__(64) void attn_window_combine_kernel(
         const float* __restrict__ part_ml, const float* __restrict__ part_o, T* __restrict__ out, int out_stride,
@@ -429,6 +404,150 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
     }
 }
 
+// Steps of single tokens, the partial results: one wave a block of 64 keys of a row's window
+// and all G query heads of a key/value head, nothing staged.  Scores with a key a lane (the
+// key's row read straight from the cache, 16 bytes at a time; the query rows are the same address
+// for all lanes), the weights through the wave's own LDS rows, sums with a value feature a lane
+// (up to four) over the positions of a feature, 16 bytes at a time.  Same partial results and the
+// same arithmetic, term for term, as a block of keys in attn_window_kernel.
+constexpr int AD_KEYS = 64;
+
+template <typename T, int NC>
+__global__ __launch_bounds__(256) void attn_window_decode_kernel(
+        const T* __restrict__ q, int q_stride, const T* __restrict__ kc, const T* __restrict__ vc,
+        const int* __restrict__ table, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ q_start,
+        const int* __restrict__ kv_lens, int H, int Hkv, int dk, int dv, int page, float scale, int window, int slots,
+        float* __restrict__ part_ml, float* __restrict__ part_o) {
+    extern __shared__ __align__(16) float lds[];       // [4 waves][G][64] weights
+    const int b = blockIdx.z, g = blockIdx.y, G = H / Hkv;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = cu_q[b];
+    if (cu_q[b + 1] - t <= 0) return;                  // a row without a token
+    const int p = q_start[b];
+    const int visible = min(kv_lens[b], p + 1);
+    const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
+    const int slot = (int)blockIdx.x * 4 + wave;
+    const int kb = j0 / AD_KEYS + slot;
+    if (slot >= slots || kb * AD_KEYS >= visible) return;
+    float* Ps = lds + (size_t)wave * G * AD_KEYS;
+    constexpr int VL = 16 / sizeof(T);
+
+    const int j = kb * AD_KEYS + lane;
+    const bool mine = j >= j0 && j < visible;
+    long long off = -1;
+    if (mine) {
+        const int pid = table[(size_t)b * max_blocks + j / page];
+        if (pid >= 0) off = ((long long)pid * Hkv + g) * page + j % page;
+    }
+    const T* kr = off >= 0 ? kc + (size_t)off * dk : nullptr;
+    const T* qrow = q + (size_t)t * q_stride + (size_t)g * G * dk;
+    const size_t at0 = ((size_t)t * H + (size_t)g * G) * slots + slot;      // + head * slots
+    const bool kvec = dk % VL == 0;
+    for (int h0 = 0; h0 < G; h0 += 4) {
+        float s[4] = {0.f, 0.f, 0.f, 0.f};
+        if (kvec) {
+            for (int dd = 0; dd < dk; dd += VL) {
+                float kf[VL];
+#pragma unroll
+                for (int u = 0; u < VL; ++u) kf[u] = 0.f;
+                if (kr) ld_vec16(kr + dd, kf);
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb) {
+                    if (h0 + rb >= G) break;
+                    float qf[VL];
+                    ld_vec16(qrow + (size_t)(h0 + rb) * dk + dd, qf);
+#pragma unroll
+                    for (int u = 0; u < VL; ++u) s[rb] = fmaf(qf[u], kf[u], s[rb]);
+                }
+            }
+        } else {
+            for (int dd = 0; dd < dk; ++dd) {
+                const float kf = kr ? ld_f32(kr + dd) : 0.f;
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb)
+                    if (h0 + rb < G) s[rb] = fmaf(ld_f32(qrow + (size_t)(h0 + rb) * dk + dd), kf, s[rb]);
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            if (h0 + rb >= G) break;
+            float m_b, l_b;
+            Ps[(h0 + rb) * AD_KEYS + lane] = aw_block_scores(s[rb], mine, scale, m_b, l_b);
+            if (lane == 0) {
+                float* dst = part_ml + (at0 + (size_t)(h0 + rb) * slots) * 2;
+                dst[0] = m_b;
+                dst[1] = l_b;
+            }
+        }
+    }
+    __builtin_amdgcn_wave_barrier();                   // the wave's own weights are in LDS (LDS keeps a wave's order)
+    const bool vvec = page % VL == 0;
+    for (int h0 = 0; h0 < G; h0 += 4) {
+        float acc[4][NC];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) acc[rb][c] = 0.f;
+        for (int jj = 0; jj < AD_KEYS; jj += VL) {
+            const int key = kb * AD_KEYS + jj;         // VL keys of one page where pages allow
+            if (key >= visible) break;
+            float v[VL][NC];
+#pragma unroll
+            for (int u = 0; u < VL; ++u)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) v[u][c] = 0.f;
+            if (vvec) {
+                const int pid = key + VL > j0 ? table[(size_t)b * max_blocks + key / page] : -1;
+                if (pid >= 0) {
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) {
+                        const int d = lane + 64 * c;
+                        if (d < dv) {
+                            float f[VL];
+                            ld_vec16(vc + (((size_t)pid * Hkv + g) * dv + d) * page + key % page, f);
+#pragma unroll
+                            for (int u = 0; u < VL; ++u) v[u][c] = (key + u >= j0 && key + u < visible) ? f[u] : 0.f;
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < VL; ++u) {
+                    const int ku = key + u;
+                    if (ku < j0 || ku >= visible) continue;
+                    const int pid = table[(size_t)b * max_blocks + ku / page];
+                    if (pid < 0) continue;
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) {
+                        const int d = lane + 64 * c;
+                        if (d < dv) v[u][c] = ld_f32(vc + (((size_t)pid * Hkv + g) * dv + d) * page + ku % page);
+                    }
+                }
+            }
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                if (h0 + rb >= G) break;
+#pragma unroll
+                for (int u = 0; u < VL; ++u) {
+                    const float pv = Ps[(h0 + rb) * AD_KEYS + jj + u];
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) acc[rb][c] = fmaf(pv, v[u][c], acc[rb][c]);
+                }
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            if (h0 + rb >= G) break;
+            float* dst = part_o + (at0 + (size_t)(h0 + rb) * slots) * dv;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const int d = lane + 64 * c;
+                if (d < dv) dst[d] = acc[rb][c];
+            }
+        }
+    }
+}
+
 int aw_keys_a_block(int dk, int dv);
 
 size_t aw_lds_bytes(int dk, int dv, int NK) {
@@ -448,7 +567,7 @@ int aw_keys_a_block(int dk, int dv) {
 
 // blocks of keys the window of a single token can touch when no request is longer than max_kv_len
 int aw_slots(int dk, int dv, int window, int max_kv_len) {
-    const int NK = aw_keys_a_block(dk, dv);
+    const int NK = AD_KEYS;
     const int span = window > 0 ? min(window, max_kv_len) : max_kv_len;
     return (span + NK - 1) / NK + (window > 0 ? 1 : 0);      // a window may begin inside a block: one more
 }
@@ -508,19 +627,19 @@ int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, con
         // every row has at most one token: a tile a row, a block a block of keys, then the merge
         float* part_ml = workspace;
         float* part_o = workspace + (size_t)Tn * H * slots * 2;
-        kernel<<<dim3(num_rows, Hkv, slots), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start,
-                                                              kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin,
-                                                              v_interleaved, slots, part_ml, part_o);
+        auto part = NC == 1 ? attn_window_decode_kernel<T, 1> : NC == 2 ? attn_window_decode_kernel<T, 2>
+                  : NC == 3 ? attn_window_decode_kernel<T, 3> : attn_window_decode_kernel<T, 4>;
+        part<<<dim3((slots + 3) / 4, Hkv, num_rows), 256, sizeof(float) * 4 * G * AD_KEYS, stream>>>(
+            q, q_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, dk, dv, page, scale, window, slots, part_ml, part_o);
         auto combine = NC == 1 ? attn_window_combine_kernel<T, 1> : NC == 2 ? attn_window_combine_kernel<T, 2>
                      : NC == 3 ? attn_window_combine_kernel<T, 3> : attn_window_combine_kernel<T, 4>;
-        combine<<<dim3(H, num_rows), 64, 0, stream>>>(part_ml, part_o, out, out_stride, cu_q, q_start, kv_lens, H, dv, window, NK, slots,
+        combine<<<dim3(H, num_rows), 64, 0, stream>>>(part_ml, part_o, out, out_stride, cu_q, q_start, kv_lens, H, dv, window, AD_KEYS, slots,
                                                       vcos, vsin, v_interleaved);
         return 0;
     }
     const int tiles = (Tn + TQ - 1) / TQ + num_rows;   // at most: every request may end in a short tile
     kernel<<<dim3(tiles, Hkv), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens,
-                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved,
-                                                   0, nullptr, nullptr);
+                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved);
     return 0;
 }
 }  // namespace

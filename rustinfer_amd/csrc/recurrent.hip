@@ -334,26 +334,31 @@ extern "C" int ri_linear_scan(
 // y = o / sqrt(mean_group(o^2) + eps) * w * sigmoid(gate): the norm over groups of `group`
 // consecutive features (all of a row, or a head) that follows the walk, with the output gate.
 // o is 32-bit; gate and out are activations of `dtype` with row strides; w has n entries.
-// A wave a group.
+// A wave a group, or the whole block for a group of more than 512 features.
 // ---------------------------------------------------------------------------
 namespace {
-template <typename T, typename TW>
+// BLOCK_GROUP: the block's 256 threads share one group (large groups); else a wave a group,
+// group blockIdx.y * waves + wave.
+template <typename T, typename TW, bool BLOCK_GROUP>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(
         const float* __restrict__ o, int o_stride, int n, int group, const TW* __restrict__ w,
         const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride, float eps) {
+    __shared__ float red[16];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const float* orow = o + (size_t)t * o_stride;
-    for (int g0 = wave * group; g0 < n; g0 += nw * group) {
-        float ss = 0.f;
-        for (int i = lane; i < group; i += 64) { const float x = orow[g0 + i]; ss = fmaf(x, x, ss); }
-        ss = wave_sum(ss);
-        const float inv = 1.f / sqrtf(ss / (float)group + eps);
-        for (int i = lane; i < group; i += 64) {
-            const int c = g0 + i;
-            float y = orow[c] * inv * ld_f32(w + c);
-            if (gate) y *= sigmoidf_(ld_f32(gate + (size_t)t * gate_stride + c));
-            st_f32(out + (size_t)t * out_stride + c, y);
-        }
+    const int gidx = BLOCK_GROUP ? blockIdx.y : blockIdx.y * nw + wave;
+    const int g0 = gidx * group;
+    if (g0 >= n) return;
+    const int first = BLOCK_GROUP ? threadIdx.x : lane, step = BLOCK_GROUP ? blockDim.x : 64;
+    float ss = 0.f;
+    for (int i = first; i < group; i += step) { const float x = orow[g0 + i]; ss = fmaf(x, x, ss); }
+    ss = BLOCK_GROUP ? block_sum(ss, red) : wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)group + eps);
+    for (int i = first; i < group; i += step) {
+        const int c = g0 + i;
+        float y = orow[c] * inv * ld_f32(w + c);
+        if (gate) y *= sigmoidf_(ld_f32(gate + (size_t)t * gate_stride + c));
+        st_f32(out + (size_t)t * out_stride + c, y);
     }
 }
 }  // namespace
@@ -365,8 +370,13 @@ extern "C" int ri_gated_group_norm(const float* o, int o_stride, int T, int n, i
     RI_REQUIRE(o_stride >= n && out_stride >= n && (!gate || gate_stride >= n), "ri_gated_group_norm: row strides too small");
     if (T == 0) return 0;
     RI_REQUIRE(o && w && out, "ri_gated_group_norm: null pointer");
-    const int block = 64 * min(4, n / group);
-#define RI_GGN(TT, TW) gated_group_norm_kernel<TT, TW><<<T, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps)
+    RI_REQUIRE(T <= 2147483647 && n / group <= 65535 * 4, "ri_gated_group_norm: too many groups for the grid");
+    const int groups = n / group;
+    const bool big = group > 512;
+    const int block = big ? 256 : 64 * min(4, groups);
+    const dim3 grid(T, big ? groups : (groups + block / 64 - 1) / (block / 64));
+#define RI_GGN(TT, TW) do { if (big) gated_group_norm_kernel<TT, TW, true><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps); \
+        else gated_group_norm_kernel<TT, TW, false><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps); } while (0)
     if (dtype == RI_F32 && w_dtype == RI_F32) RI_GGN(float, float);
     else if (dtype == RI_BF16 && w_dtype == RI_F32) RI_GGN(bf16_t, float);
     else if (dtype == RI_BF16 && w_dtype == RI_BF16) RI_GGN(bf16_t, bf16_t);
