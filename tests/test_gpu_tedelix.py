@@ -38,9 +38,18 @@ CONFIGS = {
                                           rot=dict(base=10000.0, dims=4)), mlp=dict(kind="dense", ff=136)),
         dict(type="general_delta", mixer=dict(heads=1, dim=128), mlp=None),
     ]),
+    # a width and a vocabulary that are no multiples of eight, three and six query heads a key/value head
+    "R": dict(architecture="Tedelix", vocab=211, width=100, norm=dict(eps=1e-6), logit_scale=1.0, logit_softcap=8.0, layers=[
+        dict(type="attention", mixer=dict(heads=3, kv_heads=1, dim=24, vdim=40, mask=dict(size=21), scale=0.2,
+                                          rot=dict(base=500.0, dims=12)), mlp=dict(kind="dense", ff=50)),
+        dict(type="general_delta", mixer=dict(heads=5, dim=20), mlp=dict(kind="dense", ff=30)),
+        dict(type="attention", mixer=dict(heads=12, kv_heads=2, dim=16, vdim=18, mask=dict(size=64), scale=0.25,
+                                          rot=dict(base=10000.0, dims=16)), mlp=None),
+        dict(type="lightning", mixer=dict(heads=5, dim=20, vdim=12, decay=[0.9, 0.8, 0.7, 0.6, 0.5]), mlp=dict(kind="dense", ff=77)),
+    ]),
 }
-DECAY_RANK = {"P": 4, "Q": 12}
-PAGE = {"P": 8, "Q": 16}
+DECAY_RANK = {"P": 4, "Q": 12, "R": 7}
+PAGE = {"P": 8, "Q": 16, "R": 16}
 
 
 def bf16_round(a: np.ndarray) -> torch.Tensor:
@@ -219,7 +228,8 @@ def portion_kernel(request):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,G,dk,dv,rot,window,scale,inter", [
     (4, 2, 16, 24, 8, 9, 0.3, False), (3, 3, 40, 36, 40, 1, 0.2, False), (8, 1, 32, 16, 2, 33, 0.18, True),
-    (2, 2, 128, 128, 64, 70, 0.09, False), (5, 5, 72, 200, 72, 17, 0.12, False), (6, 2, 64, 64, 64, 500, 0.125, False)])
+    (2, 2, 128, 128, 64, 70, 0.09, False), (5, 5, 72, 200, 72, 17, 0.12, False), (6, 2, 64, 64, 64, 500, 0.125, False),
+    (6, 1, 24, 40, 12, 21, 0.2, False), (2, 1, 256, 256, 256, 40, 0.06, False)])
 def test_window_attention_alone(dtype, H, G, dk, dv, rot, window, scale, inter, portion_kernel):
     from rustinfer_amd.parts import RotaryEmbedding, WindowAttention
     d = 48
@@ -350,7 +360,7 @@ LENGTHS = (70, 3, 121, 1, 38)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q"])
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
 def test_every_cut_gives_the_plain_logits(tdirs, plain_logits, name, dtype):
     reqs, logits = plain_logits(name, LENGTHS, 21)
     eng = engine_for(tdirs[name], dtype, name)
