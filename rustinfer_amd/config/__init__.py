@@ -1,4 +1,5 @@
-from .model_config import (ConfigError, GeneralDeltaSpec, LightningSpec, LlamaConfig, ModelConfig, RopeScaling,
+from .model_config import (BeloraxConfig, BeloraxLayer, ConfigError, FeedForwardSpec, GeneralDeltaSpec, LatentAttentionSpec,
+                           NormedAttentionSpec, RetentionSpec, YarnScaling, LightningSpec, LlamaConfig, ModelConfig, RopeScaling,
                            TedelixConfig, TedelixLayer, WindowAttentionSpec, read_config_json)
 from .registry import (ArchitectureEntry, load_model_config, register_architecture,
                        registered_architectures, resolve_architecture, unregister_architecture)

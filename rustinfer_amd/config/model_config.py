@@ -441,3 +441,277 @@ class TedelixConfig(ModelConfig):
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
         return d
+
+
+# ---------------------------------------------------------------------------
+# Belorax: layers listed one by one; the norm sits on each sub-layer's output
+# ---------------------------------------------------------------------------
+@dataclass(frozen=True)
+class YarnScaling:
+    """Rotary frequencies stretched band by band: pairs that turn more than ``fast`` times over
+    ``original`` positions keep their frequency, pairs that turn fewer than ``slow`` times have it
+    divided by ``factor``, a linear ramp over the pair index between; cos and sin are multiplied by
+    ``0.1 ln(factor) + 1``."""
+    factor: float
+    original: int
+    fast: float
+    slow: float
+
+    @staticmethod
+    def from_dict(d: Dict[str, Any], where: str) -> "YarnScaling":
+        s = YarnScaling(factor=_require(d, "factor", float, where), original=_require(d, "original", int, where),
+                        fast=_require(d, "fast", float, where), slow=_require(d, "slow", float, where))
+        if not (s.factor > 0 and s.original > 0 and s.fast > 0 and s.slow > 0):
+            raise ConfigError(f"{where}: factor, original, fast and slow must be > 0")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"factor": self.factor, "original": self.original, "fast": self.fast, "slow": self.slow}
+
+
+def _rot_of(m: Dict[str, Any], where: str):
+    """(base, dims, scaling) of a mixer's 'rot' object."""
+    rot = _obj(m, "rot", where)
+    base, dims = _require(rot, "base", float, where + ".rot"), _require(rot, "dims", int, where + ".rot")
+    sc = rot.get("scaling")
+    if sc is not None and not isinstance(sc, dict):
+        raise ConfigError(f"{where}.rot: 'scaling' must be an object or null")
+    if not base > 0 or dims <= 0 or dims % 2:
+        raise ConfigError(f"{where}.rot: base must be > 0 and dims even and > 0")
+    return base, dims, (YarnScaling.from_dict(sc, where + ".rot.scaling") if sc is not None else None)
+
+
+def _rot_dict(base, dims, scaling=None) -> Dict[str, Any]:
+    d = {"base": base, "dims": dims}
+    if scaling is not None:
+        d["scaling"] = scaling.to_dict()
+    return d
+
+
+@dataclass(frozen=True)
+class NormedAttentionSpec:
+    """Mixer ``attention``: grouped softmax attention over all earlier positions, queries and keys
+    normed head by head, no rotation, a query temperature that grows with the position's logarithm;
+    ``kv_from``: the layer whose keys and values this one reads instead of making its own."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    temp_coef: float = 0.0
+    temp_every: int = 0           # 0: no temperature
+    kv_from: Optional[int] = None
+    kind: str = "attention"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "NormedAttentionSpec":
+        temp = m.get("q_temp")
+        if temp is not None and not isinstance(temp, dict):
+            raise ConfigError(f"{where}: 'q_temp' must be an object or null")
+        kv_from = m.get("kv_from")
+        s = NormedAttentionSpec(
+            heads=_require(m, "heads", int, where), kv_heads=_require(m, "kv_heads", int, where),
+            dim=_require(m, "dim", int, where), vdim=_require(m, "vdim", int, where),
+            scale=_require(m, "scale", float, where),
+            temp_coef=_require(temp, "coef", float, where + ".q_temp") if temp is not None else 0.0,
+            temp_every=_require(temp, "every", int, where + ".q_temp") if temp is not None else 0,
+            kv_from=_typed(kv_from, "kv_from", int, where) if kv_from is not None else None)
+        if min(s.heads, s.kv_heads, s.dim, s.vdim) <= 0 or s.heads % s.kv_heads:
+            raise ConfigError(f"{where}: heads, kv_heads, dim and vdim must be > 0 and heads a multiple of kv_heads")
+        if temp is not None and s.temp_every <= 0:
+            raise ConfigError(f"{where}.q_temp: every must be > 0")
+        if s.dim > MAX_HEAD_DIM or s.vdim > MAX_HEAD_DIM or s.heads // s.kv_heads > 32:
+            raise ConfigError(f"{where}: heads of more than {MAX_HEAD_DIM} features or more than 32 query heads a "
+                              f"key/value head are beyond the attention kernels")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+        if self.temp_every > 0:
+            d["q_temp"] = {"coef": self.temp_coef, "every": self.temp_every}
+        if self.kv_from is not None:
+            d["kv_from"] = self.kv_from
+        return d
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Mixer ``latent_attention``: keys and values of all heads come from one latent vector of
+    ``kv_rank`` features a token, plus one rotated key part of ``rot_dim`` features shared by the heads."""
+    heads: int
+    dim: int                 # unrotated query/key features a head
+    rot_dim: int             # rotated query/key features a head
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot_base: float
+    rot_dims: int
+    rot_scaling: Optional[YarnScaling] = None
+    kind: str = "latent_attention"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "LatentAttentionSpec":
+        base, dims, scaling = _rot_of(m, where)
+        s = LatentAttentionSpec(
+            heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where),
+            rot_dim=_require(m, "rot_dim", int, where), vdim=_require(m, "vdim", int, where),
+            kv_rank=_require(m, "kv_rank", int, where), scale=_require(m, "scale", float, where),
+            rot_base=base, rot_dims=dims, rot_scaling=scaling)
+        if min(s.heads, s.dim, s.rot_dim, s.vdim, s.kv_rank) <= 0:
+            raise ConfigError(f"{where}: heads, dim, rot_dim, vdim and kv_rank must be > 0")
+        if s.rot_dims > s.rot_dim:
+            raise ConfigError(f"{where}: rot.dims {s.rot_dims} exceeds rot_dim {s.rot_dim}")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim, "kv_rank": self.kv_rank,
+                "scale": self.scale, "rot": _rot_dict(self.rot_base, self.rot_dims, self.rot_scaling)}
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Mixer ``retention``: linear attention with one fixed decay a head, rotated queries and keys."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    rot_base: float
+    rot_dims: int
+    kind: str = "retention"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "RetentionSpec":
+        decay = m.get("decay")
+        if not isinstance(decay, list):
+            raise ConfigError(f"{where}: 'decay' must be a list with one number for each head")
+        base, dims, scaling = _rot_of(m, where)
+        if scaling is not None:
+            raise ConfigError(f"{where}.rot: this mixer's rotation takes no scaling")
+        s = RetentionSpec(heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where),
+                          vdim=_require(m, "vdim", int, where),
+                          decay=tuple(_typed(x, "decay", float, where) for x in decay), rot_base=base, rot_dims=dims)
+        if min(s.heads, s.dim, s.vdim) <= 0 or len(s.decay) != s.heads:
+            raise ConfigError(f"{where}: heads, dim, vdim must be > 0 and 'decay' hold {s.heads} numbers")
+        if s.dim > MAX_HEAD_DIM or s.rot_dims > s.dim:
+            raise ConfigError(f"{where}: dim {s.dim} exceeds {MAX_HEAD_DIM}, the most key rows the state kernel takes, "
+                              f"or rot.dims {s.rot_dims} exceeds dim")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "decay": list(self.decay),
+                "rot": _rot_dict(self.rot_base, self.rot_dims)}
+
+
+BELORAX_MIXERS = {"attention": NormedAttentionSpec, "latent_attention": LatentAttentionSpec, "retention": RetentionSpec}
+
+
+@dataclass(frozen=True)
+class FeedForwardSpec:
+    """``dense``: one gated feed-forward of width ``ff``.  ``moe``: ``experts`` of them of width ``ff``
+    each, of which a token uses ``top``."""
+    kind: str
+    ff: int
+    experts: int = 0
+    top: int = 0
+
+    @staticmethod
+    def from_dict(mlp: Dict[str, Any], where: str) -> "FeedForwardSpec":
+        kind = _require(mlp, "kind", str, where)
+        if kind == "dense":
+            s = FeedForwardSpec("dense", _require(mlp, "ff", int, where))
+        elif kind == "moe":
+            router = _obj(mlp, "router", where)
+            s = FeedForwardSpec("moe", _require(_obj(mlp, "expert", where), "ff", int, where + ".expert"),
+                                _require(router, "experts", int, where + ".router"), _require(router, "top", int, where + ".router"))
+            if not (0 < s.top <= s.experts):
+                raise ConfigError(f"{where}.router: need 0 < top <= experts")
+        else:
+            raise ConfigError(f"{where}: unknown feed-forward kind {kind!r} (known: dense, moe)")
+        if s.ff <= 0:
+            raise ConfigError(f"{where}: ff must be > 0")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff}
+        return {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
+
+
+@dataclass(frozen=True)
+class BeloraxLayer:
+    mixer: Any                                # one of the specs above
+    mlp: Optional[FeedForwardSpec] = None     # None: the layer has no feed-forward
+
+    @property
+    def type(self) -> str:
+        return self.mixer.kind
+
+
+@dataclass(frozen=True)
+class BeloraxConfig(ModelConfig):
+    """``{"architecture": "Belorax", "vocab", "width", "norm": {"eps"}, "embedding": {"scale"},
+    "residual_mult", "layers": [{"type", "mixer": {...}, "mlp": {...} | null}]}``.  Each sub-layer
+    reads the residual stream itself and its output is normed before it is added, times
+    ``residual_mult``; the head has a matrix of its own; no end-of-sequence token of its own."""
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    norm_eps: float = 1e-6
+    embedding_scale: float = 1.0
+    residual_mult: float = 1.0
+    layers: tuple = ()
+    eos_token_ids: tuple = ()
+    architecture: str = "Belorax"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "BeloraxConfig":
+        layers_in = d.get("layers")
+        if not isinstance(layers_in, list) or not layers_in:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(layers_in):
+            w = f"{where}.layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{w}: must be an object")
+            kind = _require(entry, "type", str, w)
+            if kind not in BELORAX_MIXERS:
+                raise ConfigError(f"{w}: unknown mixer type {kind!r} (known: {', '.join(sorted(BELORAX_MIXERS))})")
+            mixer = BELORAX_MIXERS[kind].from_dict(_obj(entry, "mixer", w), w + ".mixer")
+            mlp = entry.get("mlp")
+            if mlp is not None and not isinstance(mlp, dict):
+                raise ConfigError(f"{w}: 'mlp' must be null or an object")
+            layers.append(BeloraxLayer(mixer, FeedForwardSpec.from_dict(mlp, w + ".mlp") if mlp is not None else None))
+        for i, layer in enumerate(layers):
+            j = getattr(layer.mixer, "kv_from", None)
+            if j is None:
+                continue
+            w = f"{where}.layers[{i}].mixer"
+            if not (0 <= j < i) or not isinstance(layers[j].mixer, NormedAttentionSpec) or layers[j].mixer.kv_from is not None:
+                raise ConfigError(f"{w}: kv_from must name an earlier attention layer that has keys and values of its own")
+            a, b = layer.mixer, layers[j].mixer
+            if (a.kv_heads, a.dim, a.vdim) != (b.kv_heads, b.dim, b.vdim):
+                raise ConfigError(f"{w}: kv_heads, dim and vdim must equal those of layer {j}, whose keys and values it reads")
+        eos = d.get("eos_token_id")
+        eos_ids = () if eos is None else tuple(_typed(e, "eos_token_id", int, where) for e in (eos if isinstance(eos, list) else [eos]))
+        emb = d.get("embedding")
+        if emb is not None and not isinstance(emb, dict):
+            raise ConfigError(f"{where}: 'embedding' must be an object")
+        cfg = cls(vocab_size=_require(d, "vocab", int, where), hidden_size=_require(d, "width", int, where),
+                  norm_eps=_require(_obj(d, "norm", where), "eps", float, where + ".norm"),
+                  embedding_scale=_typed(emb.get("scale", 1.0), "scale", float, where + ".embedding") if emb else 1.0,
+                  residual_mult=_typed(d.get("residual_mult", 1.0), "residual_mult", float, where),
+                  layers=tuple(layers), eos_token_ids=eos_ids)
+        if cfg.vocab_size <= 0 or cfg.hidden_size <= 0 or not cfg.norm_eps > 0:
+            raise ConfigError(f"{where}: vocab and width must be > 0, norm.eps > 0")
+        return cfg
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {
+            "architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+            "norm": {"eps": self.norm_eps}, "embedding": {"scale": self.embedding_scale},
+            "residual_mult": self.residual_mult,
+            "layers": [{"type": l.type, "mixer": l.mixer.to_dict(), "mlp": None if l.mlp is None else l.mlp.to_dict()}
+                       for l in self.layers]}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

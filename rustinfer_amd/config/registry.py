@@ -101,3 +101,4 @@ def _ensure_builtin() -> None:
     _builtin_done = True
     from ..models import llama  # noqa: F401  (registers LlamaForCausalLM)
     from ..models import tedelix  # noqa: F401  (registers Tedelix)
+    from ..models import belorax  # noqa: F401  (registers Belorax)

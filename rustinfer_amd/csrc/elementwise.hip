@@ -7,33 +7,41 @@
 // ---------------------------------------------------------------------------
 // A negative id -(k+1) stands for device_tokens[k]: the token a previous step sampled and left
 // on the device, so that the next step can start before the host has seen it.
-template <typename TW>
+template <typename TW, typename TO>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ device_tokens,
-                             const TW* __restrict__ table, float* __restrict__ x, int d, int V) {
+                             const TW* __restrict__ table, float* __restrict__ x, int d, int V, float scale,
+                             TO* __restrict__ act) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 && device_tokens != nullptr) id = device_tokens[-1 - id];
     float* xr = x + (size_t)t * d;
+    TO* ar = act ? act + (size_t)t * d : nullptr;
     if (id < 0 || id >= V) {
-        for (int i = threadIdx.x; i < d; i += blockDim.x) xr[i] = 0.f;
+        for (int i = threadIdx.x; i < d; i += blockDim.x) { xr[i] = 0.f; if (ar) st_f32(ar + i, 0.f); }
         return;
     }
     const TW* row = table + (size_t)id * d;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) xr[i] = ld_f32(row + i);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = ld_f32(row + i) * scale;
+        xr[i] = v;
+        if (ar) st_f32(ar + i, v);
+    }
 }
 
+// scale: every row is multiplied by it (1: the table's rows as they are).  act: null, or [T][d] of
+// act_dtype that takes the same rows rounded (what a sub-layer that reads the stream itself is given).
 extern "C" int ri_embed(const int* ids, const int* device_tokens, const void* table, int table_dtype,
-                        float* x, int T, int d, int V, hipStream_t stream) {
+                        float* x, int T, int d, int V, float scale, void* act, int act_dtype, hipStream_t stream) {
     RI_REQUIRE(T >= 0 && d > 0 && V > 0, "ri_embed: bad sizes T=%d d=%d V=%d", T, d, V);
     if (T == 0) return 0;
     RI_REQUIRE(ids && table && x, "ri_embed: null pointer");
     const int block = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
-    if (table_dtype == RI_F32)
-        embed_kernel<float><<<T, block, 0, stream>>>(ids, device_tokens, (const float*)table, x, d, V);
-    else if (table_dtype == RI_BF16)
-        embed_kernel<bf16_t><<<T, block, 0, stream>>>(ids, device_tokens, (const bf16_t*)table, x, d, V);
+    if (table_dtype == RI_F32 && (!act || act_dtype == RI_F32))
+        embed_kernel<float, float><<<T, block, 0, stream>>>(ids, device_tokens, (const float*)table, x, d, V, scale, (float*)act);
+    else if (table_dtype == RI_BF16 && (!act || act_dtype == RI_BF16))
+        embed_kernel<bf16_t, bf16_t><<<T, block, 0, stream>>>(ids, device_tokens, (const bf16_t*)table, x, d, V, scale, (bf16_t*)act);
     else
-        return ri_fail("ri_embed: unknown dtype %d", table_dtype);
+        return ri_fail("ri_embed: table dtype %d with a copy in dtype %d is not taken", table_dtype, act_dtype);
     RI_LAUNCHED("ri_embed");
     return 0;
 }
@@ -499,4 +507,112 @@ extern "C" int ri_scale_softcap(float* x, int rows, int cols, float scale, float
     scale_softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, n, scale, cap);
     RI_LAUNCHED("ri_scale_softcap");
     return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The norm on a sub-layer's OUTPUT, added to the residual stream:
+//   y = sum_p delta[p][r];   x[r] += mult * y * rsqrt(mean(y^2) + eps) * (one_plus ? 1 + w : w)
+// all in 32-bit.  act: null, or [rows][d] that takes the new x[r] rounded to act's dtype: the input
+// of the next sub-layer where sub-layers read the stream itself.  delta null: only that copy is made.
+// One block a row; the row's sums stay in registers between the two passes for d up to 4 * 4 * BLOCK.
+// ---------------------------------------------------------------------------
+template <typename TD, typename TW, typename TO, int BLOCK, int VEC>
+__global__ __launch_bounds__(BLOCK) void norm_residual_kernel(
+        float* __restrict__ x, const TD* __restrict__ delta, int parts, size_t part_stride, const TW* __restrict__ w,
+        int one_plus, float mult, float eps, TO* __restrict__ act, int d) {
+    __shared__ float red[16];
+    using L = VecLoad<VEC>;
+    const int r = blockIdx.x;
+    float* xr = x + (size_t)r * d;
+    TO* ar = act ? act + (size_t)r * d : nullptr;
+    if (!delta) {
+        for (int i = threadIdx.x * VEC; i < d; i += BLOCK * VEC) { float v[VEC]; L::ld(xr + i, v); L::st(ar + i, v); }
+        return;
+    }
+    const TD* dr = delta + (size_t)r * d;
+    constexpr int CACHE = 4;
+    float y[CACHE][VEC];
+    float ss = 0.f;
+    auto sum_at = [&](int i, float* v) {
+        L::ld(dr + i, v);
+        for (int p = 1; p < parts; ++p) {
+            float t[VEC];
+            L::ld(dr + p * part_stride + i, t);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] += t[e];
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = (threadIdx.x + k * BLOCK) * VEC;
+        if (i < d) {
+            sum_at(i, y[k]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) ss = fmaf(y[k][e], y[k][e], ss);
+        }
+    }
+    for (int i = (threadIdx.x + CACHE * BLOCK) * VEC; i < d; i += BLOCK * VEC) {
+        float v[VEC];
+        sum_at(i, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) ss = fmaf(v[e], v[e], ss);
+    }
+    ss = block_sum(ss, red);
+    const float rs = mult / sqrtf(ss / (float)d + eps);
+    auto finish = [&](int i, const float* v) {
+        float xv[VEC], wv[VEC];
+        L::ld(xr + i, xv);
+        L::ld(w + i, wv);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xv[e] = fmaf(v[e] * rs, one_plus ? 1.f + wv[e] : wv[e], xv[e]);
+        L::st(xr + i, xv);
+        if (ar) L::st(ar + i, xv);
+    };
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = (threadIdx.x + k * BLOCK) * VEC;
+        if (i < d) finish(i, y[k]);
+    }
+    for (int i = (threadIdx.x + CACHE * BLOCK) * VEC; i < d; i += BLOCK * VEC) {
+        float v[VEC];
+        sum_at(i, v);
+        finish(i, v);
+    }
+}
+
+template <typename TD, typename TW, typename TO>
+static int launch_norm_residual(float* x, const void* delta, int parts, size_t ps, const void* w, int one_plus, float mult,
+                                float eps, void* act, int rows, int d, hipStream_t stream) {
+#define RI_NR(BLOCK, VEC) norm_residual_kernel<TD, TW, TO, BLOCK, VEC><<<rows, BLOCK, 0, stream>>>( \
+        x, (const TD*)delta, parts, ps, (const TW*)w, one_plus, mult, eps, (TO*)act, d)
+    if (d % 4 == 0) { if (d <= 2048) RI_NR(128, 4); else RI_NR(256, 4); }
+    else RI_NR(256, 1);
+#undef RI_NR
+    RI_LAUNCHED("ri_norm_residual");
+    return 0;
+}
+
+// delta: null, or [parts][rows][d] of delta_dtype (a stack of partial sums must be 32-bit).
+extern "C" int ri_norm_residual(float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
+                                const void* w, int w_dtype, int one_plus, float mult, float eps,
+                                void* act, int act_dtype, int rows, int d, hipStream_t stream) {
+    RI_REQUIRE(rows >= 0 && d > 0, "ri_norm_residual: bad sizes rows=%d d=%d", rows, d);
+    if (rows == 0) return 0;
+    RI_REQUIRE(x && (delta || act), "ri_norm_residual: null pointer");
+    RI_REQUIRE(!delta || (w && eps > 0.f && parts >= 1 && part_stride >= 0), "ri_norm_residual: a delta needs a weight, eps > 0 and parts >= 1");
+    RI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)act % 16 == 0,
+               "ri_norm_residual: operands must be 16-byte aligned");
+    RI_REQUIRE(d % 4 != 0 || part_stride % 4 == 0, "ri_norm_residual: part stride must be a multiple of 4");
+    RI_REQUIRE(parts <= 1 || delta_dtype == RI_F32, "ri_norm_residual: partial sums must be 32-bit");
+    if (!delta) { delta_dtype = RI_F32; w_dtype = RI_F32; }
+    if (!act) act_dtype = RI_F32;
+    const size_t ps = (size_t)part_stride;
+#define RI_NR_CASE(DD, TD, WD, TW, AD, TO) if (delta_dtype == DD && w_dtype == WD && act_dtype == AD) \
+        return launch_norm_residual<TD, TW, TO>(x, delta, parts, ps, w, one_plus, mult, eps, act, rows, d, stream)
+    RI_NR_CASE(RI_F32, float, RI_F32, float, RI_F32, float);
+    RI_NR_CASE(RI_F32, float, RI_F32, float, RI_BF16, bf16_t);
+    RI_NR_CASE(RI_BF16, bf16_t, RI_F32, float, RI_BF16, bf16_t);
+    RI_NR_CASE(RI_BF16, bf16_t, RI_F32, float, RI_F32, float);
+#undef RI_NR_CASE
+    return ri_fail("ri_norm_residual: unsupported dtypes delta=%d weight=%d act=%d", delta_dtype, w_dtype, act_dtype);
 }

@@ -38,6 +38,11 @@ struct ScanArgs {
     const int *cu_q, *q_start, *slots;
     int H, dk, dv, P, silu_in;
     float unit_eps, decay_c;
+    // the decay form's rotation of r and k by the token's position over their first `rot` features
+    // (feature i with i + rot/2; tables [positions][rot/2], null: none), and a factor on k after it
+    const float *rot_cos, *rot_sin;
+    int rot;
+    float k_scale;
 };
 
 // exp on the hardware's 2^x (an error of a unit or two in the last place of 32 bits) and a division
@@ -80,7 +85,7 @@ __device__ __forceinline__ float wave_sum_rows(float x) {
            + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 48))));
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL>
+template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT>
 __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) {
     constexpr int SC_EPL = EPL;
     extern __shared__ __align__(16) float lds[];
@@ -111,6 +116,10 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
     // what this thread stages of a stretch: asked for a stretch ahead, so that the walk hides the wait
     float raw_r[TPW][SC_EPL], raw_k[TPW][SC_EPL], raw_w[DELTA ? TPW : 1][SC_EPL], raw_a[DELTA ? TPW : 1][SC_EPL];
     float raw_v[SC_CH];
+    // ROT: the rotation partners of r and k (feature idx +- rot/2), asked for with them
+    float part_r[ROT ? TPW : 1][SC_EPL], part_k[ROT ? TPW : 1][SC_EPL];
+    const int rot_half = ROT ? a.rot >> 1 : 0;
+    const int pos0 = ROT ? a.q_start[b] : 0;
     auto ask = [&](int c0) {
         const int nc = min(SC_CH, n - c0);
 #pragma unroll
@@ -124,6 +133,12 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                 const int c = h * dk + (on ? idx : 0);
                 raw_r[i][e] = on ? ld_f32(rp + t * a.r_stride + c) : 0.f;
                 raw_k[i][e] = on ? ld_f32(kp + t * a.k_stride + c) : 0.f;
+                if (ROT) {
+                    const bool turn = on && idx < a.rot;
+                    const int cp = turn ? (idx < rot_half ? c + rot_half : c - rot_half) : c;
+                    part_r[i][e] = turn ? ld_f32(rp + t * a.r_stride + cp) : 0.f;
+                    part_k[i][e] = turn ? ld_f32(kp + t * a.k_stride + cp) : 0.f;
+                }
                 if (DELTA) {
                     raw_w[i][e] = on ? ld_f32(wlp + t * a.wl_stride + c) : 0.f;
                     raw_a[i][e] = on ? ld_f32(alp + t * a.al_stride + c) : 0.f;
@@ -138,7 +153,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
             raw_v[e] = (x < nc * CPB && jj < dv) ? ld_f32(vp + (size_t)(t_lo + c0 + tt) * a.v_stride + h * dv + jj) : 0.f;
         }
     };
-    auto stage = [&](float* buf, int nc) {
+    auto stage = [&](float* buf, int nc, int c0) {
         float* rs = buf;                               // [SC_CH][DKP] each
         float* ks = rs + SC_CH * DKP;
         float* us = ks + SC_CH * DKP;                  // the delta form's three
@@ -176,6 +191,15 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                     if (idx >= DKP) continue;
                     float r = raw_r[i][e], k = raw_k[i][e];
                     if (a.silu_in && idx < dk) { r = siluf_(r); k = siluf_(k); }
+                    if (ROT) {
+                        if (idx < a.rot) {
+                            const size_t at = (size_t)(pos0 + c0 + tt) * rot_half + (idx < rot_half ? idx : idx - rot_half);
+                            const float cs = a.rot_cos[at], sn = idx < rot_half ? -a.rot_sin[at] : a.rot_sin[at];
+                            r = fmaf(part_r[i][e], sn, r * cs);
+                            k = fmaf(part_k[i][e], sn, k * cs);
+                        }
+                        k *= a.k_scale;
+                    }
                     rs[tt * DKP + idx] = r; ks[tt * DKP + idx] = k;
                 }
             }
@@ -194,7 +218,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         float* buf = lds + turn * BUF;
         // the other buffer may still be walked by a slower wave; this one was last walked two
         // stretches ago, before the barrier of the last stretch
-        stage(buf, nc);
+        stage(buf, nc, c0);
         if (c0 + SC_CH < n) ask(c0 + SC_CH);
         lds_barrier();
         const float* rs = buf;
@@ -252,12 +276,12 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
     }
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL>
-int launch_scan_as(const ScanArgs& a, int num_rows, hipStream_t stream) {
+template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT>
+int launch_scan_rot(const ScanArgs& a, int num_rows, hipStream_t stream) {
     const int P = a.P, DKP = P * R, CPB = NW * (64 / P);
     const size_t lds = sizeof(float) * 2 * ((DELTA ? 5 : 2) * SC_CH * DKP + SC_CH * CPB);
     dim3 grid((a.dv + CPB - 1) / CPB, a.H, num_rows);
-    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL>;
+    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL, ROT>;
     if (lds > 64 * 1024) {
         // more LDS than a kernel gets unasked (the delta form with more than 128 key rows)
         static bool asked = false;
@@ -269,6 +293,14 @@ int launch_scan_as(const ScanArgs& a, int num_rows, hipStream_t stream) {
     }
     kernel<<<grid, NW * 64, lds, stream>>>(a);
     return 0;
+}
+
+template <typename T, bool DELTA, int R, int NW, int EPL>
+int launch_scan_as(const ScanArgs& a, int num_rows, hipStream_t stream) {
+    if constexpr (!DELTA) {
+        if (a.rot_cos != nullptr || a.k_scale != 1.f) return launch_scan_rot<T, DELTA, R, NW, EPL, true>(a, num_rows, stream);
+    }
+    return launch_scan_rot<T, DELTA, R, NW, EPL, false>(a, num_rows, stream);
 }
 
 template <typename T, bool DELTA, int R>
@@ -299,7 +331,8 @@ extern "C" int ri_linear_scan(
         const float* w0, const float* ab, const float* decay, int delta, int silu_in,
         float unit_eps, float decay_c, float* state, int num_slots, float* out, int out_stride,
         const int* cu_q, const int* q_start, const int* slots, int num_rows, int T,
-        int H, int dk, int dv, hipStream_t stream) {
+        int H, int dk, int dv, const float* rot_cos, const float* rot_sin, int rot, int rot_rows, int max_position,
+        float k_scale, hipStream_t stream) {
     RI_REQUIRE(H > 0 && dk > 0 && dv > 0 && dk <= 256, "ri_linear_scan: bad sizes H=%d dk=%d dv=%d (dk <= 256)", H, dk, dv);
     RI_REQUIRE(num_rows >= 0 && T >= 0 && num_slots > 0, "ri_linear_scan: bad counts");
     RI_REQUIRE(r_stride >= H * dk && k_stride >= H * dk && v_stride >= H * dv && out_stride >= H * dv,
@@ -309,6 +342,9 @@ extern "C" int ri_linear_scan(
     RI_REQUIRE(H <= 65535 && num_rows <= 65535, "ri_linear_scan: too many heads or rows for the grid");
     if (delta) RI_REQUIRE(wl && al && w0 && ab && wl_stride >= H * dk && al_stride >= H * dk, "ri_linear_scan: the delta form needs wl, al, w0, ab");
     else RI_REQUIRE(decay, "ri_linear_scan: the decay form needs a decay for each head");
+    if (rot_cos) RI_REQUIRE(!delta && !silu_in && rot_sin && rot > 0 && rot % 2 == 0 && rot <= dk && rot_rows > 0 && max_position < rot_rows,
+                            "ri_linear_scan: a rotation goes with the decay form without silu, an even rot <= dk and tables of %d positions (got %d rows)", max_position + 1, rot_rows);
+    if (delta) RI_REQUIRE(!rot_cos && k_scale == 1.f, "ri_linear_scan: the delta form takes no rotation and no key factor");
     // key rows a thread: 8, or 16 where 8 would need more than the 16 lanes a column may have
     const int R = dk <= 128 ? 8 : 16;
     int P = 1;
@@ -319,6 +355,7 @@ extern "C" int ri_linear_scan(
     a.w0 = w0; a.ab = ab; a.decay = decay; a.state = state; a.out = out; a.out_stride = out_stride;
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = silu_in; a.unit_eps = unit_eps; a.decay_c = decay_c;
+    a.rot_cos = rot_cos; a.rot_sin = rot_sin; a.rot = rot_cos ? rot : 0; a.k_scale = k_scale;
     int rc;
 #define RI_SCAN(TT, DD) (R == 8 ? launch_scan<TT, DD, 8>(a, num_rows, stream) : launch_scan<TT, DD, 16>(a, num_rows, stream))
     if (dtype == RI_F32) rc = delta ? RI_SCAN(float, true) : RI_SCAN(float, false);
@@ -331,7 +368,8 @@ extern "C" int ri_linear_scan(
 }
 
 // ---------------------------------------------------------------------------
-// y = o / sqrt(mean_group(o^2) + eps) * w * sigmoid(gate): the norm over groups of `group`
+// y = o / sqrt(mean_group(o^2) + eps) * w * sigmoid(gate) (w null: no weight; gate_silu: silu(gate)
+// in place of the sigmoid): the norm over groups of `group`
 // consecutive features (all of a row, or a head) that follows the walk, with the output gate.
 // o is 32-bit; gate and out are activations of `dtype` with row strides; w has n entries.
 // A wave a group, or the whole block for a group of more than 512 features.
@@ -342,7 +380,7 @@ namespace {
 template <typename T, typename TW, bool BLOCK_GROUP>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(
         const float* __restrict__ o, int o_stride, int n, int group, const TW* __restrict__ w,
-        const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride, float eps) {
+        const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride, float eps, int gate_silu) {
     __shared__ float red[16];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const float* orow = o + (size_t)t * o_stride;
@@ -356,8 +394,12 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     const float inv = 1.f / sqrtf(ss / (float)group + eps);
     for (int i = first; i < group; i += step) {
         const int c = g0 + i;
-        float y = orow[c] * inv * ld_f32(w + c);
-        if (gate) y *= sigmoidf_(ld_f32(gate + (size_t)t * gate_stride + c));
+        float y = orow[c] * inv;
+        if (w) y *= ld_f32(w + c);
+        if (gate) {
+            const float z = ld_f32(gate + (size_t)t * gate_stride + c);
+            y *= gate_silu ? siluf_(z) : sigmoidf_(z);
+        }
         st_f32(out + (size_t)t * out_stride + c, y);
     }
 }
@@ -365,18 +407,19 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
 
 extern "C" int ri_gated_group_norm(const float* o, int o_stride, int T, int n, int group, const void* w, int w_dtype,
                                    const void* gate, int gate_stride, void* out, int out_stride, int dtype,
-                                   float eps, hipStream_t stream) {
+                                   float eps, int gate_silu, hipStream_t stream) {
     RI_REQUIRE(T >= 0 && n > 0 && group > 0 && n % group == 0, "ri_gated_group_norm: %d features do not split into groups of %d", n, group);
     RI_REQUIRE(o_stride >= n && out_stride >= n && (!gate || gate_stride >= n), "ri_gated_group_norm: row strides too small");
     if (T == 0) return 0;
-    RI_REQUIRE(o && w && out, "ri_gated_group_norm: null pointer");
+    RI_REQUIRE(o && out, "ri_gated_group_norm: null pointer");
+    if (!w) w_dtype = RI_F32;
     RI_REQUIRE(T <= 2147483647 && n / group <= 65535 * 4, "ri_gated_group_norm: too many groups for the grid");
     const int groups = n / group;
     const bool big = group > 512;
     const int block = big ? 256 : 64 * min(4, groups);
     const dim3 grid(T, big ? groups : (groups + block / 64 - 1) / (block / 64));
-#define RI_GGN(TT, TW) do { if (big) gated_group_norm_kernel<TT, TW, true><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps); \
-        else gated_group_norm_kernel<TT, TW, false><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps); } while (0)
+#define RI_GGN(TT, TW) do { if (big) gated_group_norm_kernel<TT, TW, true><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps, gate_silu); \
+        else gated_group_norm_kernel<TT, TW, false><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps, gate_silu); } while (0)
     if (dtype == RI_F32 && w_dtype == RI_F32) RI_GGN(float, float);
     else if (dtype == RI_BF16 && w_dtype == RI_F32) RI_GGN(bf16_t, float);
     else if (dtype == RI_BF16 && w_dtype == RI_BF16) RI_GGN(bf16_t, bf16_t);

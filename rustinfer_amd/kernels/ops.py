@@ -102,9 +102,11 @@ def _rows2d(t: torch.Tensor, name: str):
 
 
 def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor,
-          device_tokens: Optional[torch.Tensor] = None) -> None:
-    """``out_x[t] = table[ids[t]]``; an id ``-(k+1)`` means ``device_tokens[k]`` (int32, on the device)."""
-    _dev(ids, table, out_x, device_tokens)
+          device_tokens: Optional[torch.Tensor] = None, scale: float = 1.0,
+          act: Optional[torch.Tensor] = None) -> None:
+    """``out_x[t] = table[ids[t]] * scale``; an id ``-(k+1)`` means ``device_tokens[k]`` (int32, on the
+    device).  ``act`` ([T, d] in the table's dtype) takes the same rows rounded to its dtype."""
+    _dev(ids, table, out_x, device_tokens, act)
     if device_tokens is not None:
         _i32(device_tokens, "device_tokens")
     T = ids.numel()
@@ -114,7 +116,40 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor,
         raise KernelError(f"embed: out must be contiguous float32 [{T}, {d}]")
     if not table.is_contiguous():
         raise KernelError("embed: table must be contiguous")
-    _check(_lib().ri_embed(_ptr(ids), _ptr(device_tokens), _ptr(table), _dt(table), _ptr(out_x), T, d, V, _stream()))
+    if act is not None and (tuple(act.shape) != (T, d) or not act.is_contiguous() or act.dtype != table.dtype):
+        raise KernelError(f"embed: the rounded copy must be contiguous [{T}, {d}] in the table's dtype")
+    _check(_lib().ri_embed(_ptr(ids), _ptr(device_tokens), _ptr(table), _dt(table), _ptr(out_x), T, d, V,
+                           ctypes.c_float(scale), _ptr(act), _dt(act) if act is not None else 0, _stream()))
+
+
+def norm_residual(x: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float,
+                  mult: float = 1.0, one_plus: bool = False, act: Optional[torch.Tensor] = None) -> None:
+    """The norm on a sub-layer's output, added to the 32-bit residual stream in place:
+    ``x += mult * delta * rsqrt(mean(delta^2) + eps) * (1 + weight if one_plus else weight)``.
+    ``delta`` is ``[T, d]`` (activations' dtype or 32-bit) or a 32-bit stack ``[P, T, d]`` of partial
+    sums.  ``act`` ([T, d]) takes the new ``x`` rounded to its dtype; with ``delta = None`` only that
+    copy is made."""
+    _dev(x, delta, weight, act)
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("norm_residual: x must be contiguous float32")
+    parts, stride, ddt = 1, 0, F32
+    if delta is not None:
+        if delta.dim() == 3:
+            parts, stride = delta.shape[0], delta.stride(0)
+        if delta.dim() not in (2, 3) or tuple(delta.shape[-2:]) != (T, d) or delta.stride(-1) != 1 or delta.stride(-2) != d \
+                or (delta.dim() == 3 and delta.dtype != torch.float32):
+            raise KernelError("norm_residual: delta must be [T, d] or a float32 stack [P, T, d] with contiguous rows")
+        if weight is None or weight.dtype != torch.float32 or weight.numel() != d or not weight.is_contiguous():
+            raise KernelError(f"norm_residual: weight must be contiguous float32 with {d} entries")
+        ddt = _dt(delta)
+    elif act is None:
+        return
+    if act is not None and (tuple(act.shape) != (T, d) or not act.is_contiguous()):
+        raise KernelError(f"norm_residual: the rounded copy must be contiguous [{T}, {d}]")
+    _check(_lib().ri_norm_residual(_ptr(x), _ptr(delta), ddt, parts, ctypes.c_longlong(stride), _ptr(weight), F32,
+                                   int(bool(one_plus)), ctypes.c_float(mult), ctypes.c_float(eps), _ptr(act),
+                                   _dt(act) if act is not None else 0, T, d, _stream()))
 
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
@@ -961,13 +996,15 @@ def linear_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
                 H: int, dk: int, dv: int, decay: Optional[torch.Tensor] = None, silu_in: bool = False,
                 wl: Optional[torch.Tensor] = None, al: Optional[torch.Tensor] = None,
                 w0: Optional[torch.Tensor] = None, ab: Optional[torch.Tensor] = None,
-                unit_eps: float = 1e-6, decay_c: float = 1.0) -> None:
+                unit_eps: float = 1e-6, decay_c: float = 1.0, rotary=None, k_scale: float = 1.0) -> None:
     """Walk each request's tokens of the step through its state ``state[slot] [H, dk, dv]`` (32-bit):
     ``S <- diag(w) S - (a u)(u^T S) + k v^T``, ``out_t = S^T r`` (32-bit ``[T, H dv]``).
     With ``decay [H]``: ``w`` is the head's constant, no second term, and r, k, v pass through silu if
     ``silu_in``.  With ``wl, al [T, H dk]`` and 32-bit ``w0, ab [H dk]``: ``u = k / sqrt(|k|^2 + unit_eps)``,
     ``w = exp(-decay_c sigmoid(wl + w0))``, ``a = sigmoid(al + ab)``.  A request's first tokens
-    (``q_start == 0``) start from zeros."""
+    (``q_start == 0``) start from zeros.  Decay form only: ``rotary = (cos, sin, rot_dim)`` turns r and
+    k by the token's position over their first ``rot_dim`` features (feature i with i + rot_dim/2), in
+    32-bit, and ``k_scale`` multiplies k after that."""
     _dev(r, k, v, state, out, decay, wl, al, w0, ab)
     for t, name in ((r, "r"), (k, "k"), (v, "v"), (out, "out")):
         _rows2d(t, name)
@@ -990,28 +1027,159 @@ def linear_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
     _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
     _i32(ctx.q_start, "q_start", ctx.num_rows)
     _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+    rot, rcos, rsin, rrows = 0, ctypes.c_void_p(0), ctypes.c_void_p(0), 0
+    if rotary is not None:
+        rot = int(rotary[2])
+        rcos, rsin, rrows = _rot_tables(rotary, rot, "linear_scan")
     _check(_lib().ri_linear_scan(
         _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
         _ptr(wl), wl.stride(0) if wl is not None else 0, _ptr(al), al.stride(0) if al is not None else 0, _dt(r),
         _ptr(w0), _ptr(ab), _ptr(decay), int(delta), int(bool(silu_in)), ctypes.c_float(unit_eps),
         ctypes.c_float(decay_c), _ptr(state), state.shape[0], _ptr(out), out.stride(0),
-        _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.state_slots), ctx.num_rows, T, H, dk, dv, _stream()))
+        _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.state_slots), ctx.num_rows, T, H, dk, dv,
+        rcos, rsin, rot, rrows, max(int(ctx.max_kv_len) - 1, 0), ctypes.c_float(k_scale), _stream()))
 
 
-def gated_group_norm(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor,
-                     group: int, eps: float) -> None:
+def gated_group_norm(o: torch.Tensor, weight: Optional[torch.Tensor], gate: Optional[torch.Tensor], out: torch.Tensor,
+                     group: int, eps: float, gate_activation: str = "sigmoid") -> None:
     """``out = o / sqrt(mean over each group of `group` features (o^2) + eps) * weight * sigmoid(gate)``;
-    ``o`` 32-bit ``[T, n]``, ``gate`` and ``out`` activations (columns of wider buffers allowed)."""
+    ``o`` 32-bit ``[T, n]``, ``gate`` and ``out`` activations (columns of wider buffers allowed).
+    ``weight = None``: no weight; ``gate_activation = "silu"``: ``silu(gate)`` in place of the sigmoid."""
     _dev(o, weight, gate, out)
     _rows2d(o, "o")
     _rows2d(out, "out")
     T, n = o.shape
-    if o.dtype != torch.float32 or tuple(out.shape) != (T, n) or weight.numel() != n or not weight.is_contiguous():
+    if o.dtype != torch.float32 or tuple(out.shape) != (T, n) or (weight is not None and (weight.numel() != n or not weight.is_contiguous())):
         raise KernelError("gated_group_norm: 32-bit o [T, n], out [T, n] and n weights expected")
+    if gate_activation not in ("sigmoid", "silu"):
+        raise KernelError(f"gated_group_norm: unknown gate activation {gate_activation!r}")
     if gate is not None:
         _rows2d(gate, "gate")
         if tuple(gate.shape) != (T, n) or gate.dtype != out.dtype:
             raise KernelError("gated_group_norm: gate must be [T, n] in the dtype of out")
-    _check(_lib().ri_gated_group_norm(_ptr(o), o.stride(0), T, n, int(group), _ptr(weight), _dt(weight), _ptr(gate),
+    _check(_lib().ri_gated_group_norm(_ptr(o), o.stride(0), T, n, int(group), _ptr(weight),
+                                      _dt(weight) if weight is not None else F32, _ptr(gate),
                                       gate.stride(0) if gate is not None else 0, _ptr(out), out.stride(0), _dt(out),
-                                      ctypes.c_float(eps), _stream()))
+                                      ctypes.c_float(eps), int(gate_activation == "silu"), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# what some attention mixers do head by head between their projections and attention
+# ---------------------------------------------------------------------------
+def _f32_vec(t: Optional[torch.Tensor], n: int, who: str):
+    if t is not None and (t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous()):
+        raise KernelError(f"{who}: must be contiguous float32 with {n} entries")
+
+
+def head_norm_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], H: int, Hkv: int,
+                       dk: int, dv: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                       eps: float, positions: torch.Tensor, row_of_token: torch.Tensor, k_cache: torch.Tensor,
+                       v_cache: torch.Tensor, block_table: torch.Tensor, page: int, write_kv: bool = True,
+                       norm: bool = True, temp_coef: float = 0.0, temp_every: int = 0) -> None:
+    """Every head of ``q [T, H dk]`` and ``k [T, Hkv dk]`` divided by its root mean square
+    (``norm``), times a 32-bit weight of ``dk`` entries shared by the heads (or None); the query at
+    position p also times ``1 + temp_coef ln(floor((p + 1) / temp_every) + 1)`` (``temp_every > 0``).
+    q in place; k and ``v [T, Hkv dv]`` go into the token's page (``write_kv``)."""
+    _dev(q, k, v, q_weight, k_weight, positions, row_of_token, k_cache, v_cache, block_table)
+    _rows2d(q, "q")
+    T = q.shape[0]
+    if q.shape[1] != H * dk:
+        raise KernelError(f"head_norm_kv_write: q must be [T, {H * dk}]")
+    _i32(positions, "positions", T)
+    _i32(row_of_token, "row_of_token", T)
+    _f32_vec(q_weight, dk, "head_norm_kv_write: the query weight")
+    _f32_vec(k_weight, dk, "head_norm_kv_write: the key weight")
+    if write_kv:
+        _rows2d(k, "k")
+        _rows2d(v, "v")
+        if tuple(k.shape) != (T, Hkv * dk) or tuple(v.shape) != (T, Hkv * dv) or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise KernelError(f"head_norm_kv_write: k must be [T, {Hkv * dk}] and v [T, {Hkv * dv}] of {q.dtype}")
+        _check_cache_kv(k_cache, v_cache, Hkv, dk, dv, page, q.dtype, "head_norm_kv_write")
+        _i32(block_table, "block_table")
+        if block_table.dim() != 2:
+            raise KernelError("head_norm_kv_write: block_table must be [rows, max_blocks]")
+    _check(_lib().ri_head_norm_kv_write(
+        _ptr(q), q.stride(0), _ptr(k) if write_kv else ctypes.c_void_p(0), k.stride(0) if write_kv else 0,
+        _ptr(v) if write_kv else ctypes.c_void_p(0), v.stride(0) if write_kv else 0, _dt(q), T, H, Hkv, dk, dv,
+        _ptr(q_weight), _ptr(k_weight), int(bool(norm)), ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every),
+        _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0] if k_cache is not None else 0,
+        _ptr(block_table), block_table.shape[1] if block_table is not None and block_table.dim() == 2 else 0, page,
+        int(bool(write_kv)), _stream()))
+
+
+def latent_kv_write(q: torch.Tensor, down: torch.Tensor, q_abs: torch.Tensor, H: int, d: int, r: int, R: int,
+                    latent_weight: Optional[torch.Tensor], eps: float, rotary, positions: torch.Tensor,
+                    row_of_token: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    block_table: torch.Tensor, page: int, write_kv: bool = True) -> None:
+    """Attention through a latent: ``down [T, R + r]`` holds the latent's R features, which are divided
+    by their root mean square and multiplied by ``latent_weight`` (32-bit), and one rotated key part of
+    r features; the page (one key/value head) takes the key ``[latent, turned part]`` and the value
+    ``latent``.  ``q [T, H (d + r)]``: the turned rotated part of every head's query goes to the last r
+    columns of that head in ``q_abs [T, H (R + r)]``.  ``rotary = (cos, sin, rot)`` turns the first
+    ``rot`` features of a rotated part (feature i with i + rot/2)."""
+    _dev(q, down, q_abs, latent_weight, positions, row_of_token, k_cache, v_cache, block_table)
+    for t, name in ((q, "q"), (down, "down"), (q_abs, "q_abs")):
+        _rows2d(t, name)
+    T = q.shape[0]
+    if q.shape[1] != H * (d + r) or tuple(down.shape) != (T, R + r) or tuple(q_abs.shape) != (T, H * (R + r)) \
+            or down.dtype != q.dtype or q_abs.dtype != q.dtype:
+        raise KernelError(f"latent_kv_write: q [T, {H * (d + r)}], down [T, {R + r}] and q_abs [T, {H * (R + r)}] of one dtype expected")
+    _i32(positions, "positions", T)
+    _i32(row_of_token, "row_of_token", T)
+    _f32_vec(latent_weight, R, "latent_kv_write: the latent's weight")
+    rot, cos, sin, rows = 0, ctypes.c_void_p(0), ctypes.c_void_p(0), 0
+    if rotary is not None:
+        rot = int(rotary[2])
+        cos, sin, rows = _rot_tables(rotary, rot, "latent_kv_write")
+    if write_kv:
+        _check_cache_kv(k_cache, v_cache, 1, R + r, R, page, q.dtype, "latent_kv_write")
+        _i32(block_table, "block_table")
+        if block_table.dim() != 2:
+            raise KernelError("latent_kv_write: block_table must be [rows, max_blocks]")
+    _check(_lib().ri_latent_kv_write(
+        _ptr(q), q.stride(0), _ptr(down), down.stride(0), _ptr(q_abs), q_abs.stride(0), _dt(q), T, H, d, r, R, rot,
+        _ptr(latent_weight), ctypes.c_float(eps), cos, sin, rows, _ptr(positions), _ptr(row_of_token),
+        _ptr(k_cache), _ptr(v_cache), k_cache.shape[0] if k_cache is not None else 0, _ptr(block_table),
+        block_table.shape[1] if block_table is not None and block_table.dim() == 2 else 0, page, int(bool(write_kv)), _stream()))
+
+
+def head_linear(x: torch.Tensor, x_head: int, w: torch.Tensor, out: torch.Tensor, out_head: int) -> None:
+    """``out[t, h * out_head : + N] = w[h] @ x[t, h * x_head : + K]`` for every head h; ``w [H, N, K]``.
+    x and out are 2-D with unit column stride (columns of wider buffers allowed); 32-bit sums."""
+    _dev(x, w, out)
+    _rows2d(x, "x")
+    _rows2d(out, "out")
+    if w.dim() != 3 or not w.is_contiguous() or w.dtype != x.dtype or out.dtype != x.dtype or out.shape[0] != x.shape[0]:
+        raise KernelError("head_linear: w must be contiguous [H, N, K] in the dtype of x and out")
+    H, N, K = w.shape
+    if x.shape[1] < (H - 1) * x_head + K or out.shape[1] < (H - 1) * out_head + N:
+        raise KernelError("head_linear: x or out is narrower than its heads")
+    _check(_lib().ri_head_linear(_ptr(x), x.stride(0), int(x_head), _ptr(w), _ptr(out), out.stride(0), int(out_head),
+                                 _dt(x), x.shape[0], H, N, K, _stream()))
+
+
+# ---------------------------------------------------------------------------
+# a feed-forward of many experts
+# ---------------------------------------------------------------------------
+def moe_route(logits: torch.Tensor, weights: torch.Tensor, top: int, renormalize: bool = False) -> None:
+    """``weights [T, E]`` (32-bit): ``softmax(logits)`` at the ``top`` largest entries of every row (ties:
+    the lower index), 0 elsewhere; ``renormalize`` divides them by their sum."""
+    _dev(logits, weights)
+    _rows2d(logits, "logits")
+    T, E = logits.shape
+    if logits.dtype != torch.float32 or weights.dtype != torch.float32 or tuple(weights.shape) != (T, E) or not weights.is_contiguous():
+        raise KernelError("moe_route: 32-bit logits [T, E] and contiguous 32-bit weights [T, E] expected")
+    _check(_lib().ri_moe_route(_ptr(logits), logits.stride(0), _ptr(weights), T, E, int(top), int(bool(renormalize)), _stream()))
+
+
+def moe_swiglu_weighted(gate_up: torch.Tensor, weights: torch.Tensor, act: torch.Tensor, E: int, F: int) -> None:
+    """``act[t, e F + i] = weights[t, e] * silu(gate_up[t, e 2F + i]) * gate_up[t, e 2F + F + i]``."""
+    _dev(gate_up, weights, act)
+    _rows2d(gate_up, "gate_up")
+    _rows2d(act, "act")
+    T = gate_up.shape[0]
+    if gate_up.shape[1] != 2 * E * F or tuple(act.shape) != (T, E * F) or act.dtype != gate_up.dtype \
+            or weights.dtype != torch.float32 or tuple(weights.shape) != (T, E) or not weights.is_contiguous():
+        raise KernelError("moe_swiglu_weighted: gate_up [T, 2 E F], 32-bit weights [T, E] and act [T, E F] expected")
+    _check(_lib().ri_moe_swiglu_weighted(_ptr(gate_up), gate_up.stride(0), _ptr(weights), _ptr(act), act.stride(0),
+                                         _dt(act), T, E, F, _stream()))

@@ -132,6 +132,8 @@ class DecoderModel(Part):
                 layer.forward(ctx, hidden, cache, out_rows=ctx.want_rows)
             else:
                 layer.forward(ctx, hidden, cache, **kw)
+            if not getattr(layer, "leaves_act", False):
+                hidden.act = None                    # the stream has moved on; nobody has rounded it
         if W == 0:
             return ws.get("model.logits", 0, self.vocab_size, torch.float32)
         logits = ws.get("model.logits", W, self.vocab_size, torch.float32)

@@ -1,13 +1,13 @@
 from .base import (FeedForward, Mixer, Norm, PagedKVNeed, ParamSpec, Part, PositionEncoding,
                    ProjectedPart, ProjectionSet, Runtime, StateNeed, stored_to)
-from .norm import RMSNorm
+from .norm import OutputRMSNorm, RMSNorm
 from .rope import RotaryEmbedding, rotary_frequencies
 from .linear import Linear
 from .embed import Embedding, LMHead
-from .mlp import DenseMLP, SwiGLUMLP
-from .attention import PagedAttention, WindowAttention
-from .recurrent import GeneralDeltaRule, LightningAttention
-from .block import Hidden, ParallelBlock, PreNormBlock
+from .mlp import DenseMLP, MoEFeedForward, SwiGLUMLP
+from .attention import LatentAttention, PagedAttention, WindowAttention
+from .recurrent import GeneralDeltaRule, LightningAttention, Retention
+from .block import Hidden, ParallelBlock, PostNormBlock, PreNormBlock
 from .registry import (MIXERS, FEED_FORWARDS, NORMS, POSITION_ENCODINGS, register_mixer,
                        register_feed_forward, register_norm, register_position_encoding,
                        make_part)

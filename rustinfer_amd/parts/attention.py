@@ -160,16 +160,30 @@ class WindowAttention(ProjectedPart, Mixer):
     ``v_head_dim``) is applied to every value before it is cached, by the value's position, and
     undone on each head's sum by the query's position, so that a value enters the output turned by
     the distance between the two.  Scores are ``(q . k) * scale``; the softmax is over the visible
-    keys only.  Tensor names: ``q, k, v, o`` unless given."""
+    keys only.  Tensor names: ``q, k, v, o`` unless given.
+
+    ``qk_norm_eps``: queries and keys are divided by their root mean square over each head (this eps
+    inside the root) and multiplied by weights of the head's size shared by all heads (tensors
+    ``<q>.norm``, ``<k>.norm``); the cache holds the normed keys.  ``q_temperature = (coef, every)``:
+    the query at position p is multiplied by ``1 + coef ln(floor((p + 1) / every) + 1)``.  Either goes
+    without a rotation of queries and keys.  ``own_kv = False``: the layer has no keys and values of
+    its own and reads a cache that another layer writes (the run order names it)."""
 
     is_mixer = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
                  scale: float, window: Optional[int] = None, pos_enc: Optional[PositionEncoding] = None,
                  value_pos_enc: Optional[PositionEncoding] = None, interleaved_values: bool = False,
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, qk_norm_eps: Optional[float] = None,
+                 q_temperature=None, own_kv: bool = True):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        self.qk_norm_eps = float(qk_norm_eps) if qk_norm_eps is not None else None
+        self.q_temperature = (float(q_temperature[0]), int(q_temperature[1])) if q_temperature else None
+        self.own_kv = bool(own_kv)
+        self.by_head = self.qk_norm_eps is not None or self.q_temperature is not None
+        if self.by_head and (pos_enc is not None or value_pos_enc is not None):
+            raise ValueError("a norm or a temperature on queries and keys goes without a rotation")
         self.hidden_size = int(hidden_size)
         self.num_heads, self.num_kv_heads = int(num_heads), int(num_kv_heads)
         self.head_dim, self.v_head_dim = int(head_dim), int(v_head_dim)
@@ -183,8 +197,19 @@ class WindowAttention(ProjectedPart, Mixer):
 
     def in_projections(self):
         n = self.names
+        if not self.own_kv:
+            return [(n["q"], self.num_heads * self.head_dim)]
         return [(n["q"], self.num_heads * self.head_dim), (n["k"], self.num_kv_heads * self.head_dim),
                 (n["v"], self.num_kv_heads * self.v_head_dim)]
+
+    def own_specs(self):
+        if self.qk_norm_eps is None:
+            return {}
+        n = self.names
+        specs = {n["q"] + ".norm": ParamSpec((self.head_dim,), "norm")}
+        if self.own_kv:
+            specs[n["k"] + ".norm"] = ParamSpec((self.head_dim,), "norm")
+        return specs
 
     def out_projection(self):
         return (self.names["o"], self.num_heads * self.v_head_dim)
@@ -197,15 +222,119 @@ class WindowAttention(ProjectedPart, Mixer):
         if not rt.ops.window_attention_supported(self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim):
             raise ValueError(f"attention with {self.num_heads}/{self.num_kv_heads} heads of {self.head_dim} and "
                              f"{self.v_head_dim} features is beyond the window attention kernel")
+        self.q_norm_weight = self.k_norm_weight = None
+        if self.qk_norm_eps is not None:
+            f32 = lambda name: tensors[name].to(device=rt.device, dtype=torch.float32).contiguous()
+            self.q_norm_weight = f32(self.names["q"] + ".norm")
+            self.k_norm_weight = f32(self.names["k"] + ".norm") if self.own_kv else None
 
     def core(self, ctx, proj, act, cache) -> None:
         ops, n = self.rt.ops, self.names
-        q, k, v = proj[n["q"]], proj[n["k"]], proj[n["v"]]
+        q, k, v = proj[n["q"]], proj.get(n["k"]), proj.get(n["v"])
         table = ctx.block_tables[cache.group]
+        write = self.own_kv and cache.write
+        if self.by_head:
+            coef, every = self.q_temperature or (0.0, 0)
+            ops.head_norm_kv_write(q, k, v, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim,
+                                   self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps or 1.0, ctx.positions,
+                                   ctx.row_of_token, cache.k, cache.v, table, cache.page_size, write_kv=write,
+                                   norm=self.qk_norm_eps is not None, temp_coef=coef, temp_every=every)
+            ops.window_attention(q, act, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, cache.k, cache.v,
+                                 table, cache.page_size, ctx, self.scale, self.window or 0, None, False)
+            return
         rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
         vrot = self.value_pos_enc.rotary()[:2] if self.value_pos_enc is not None else None
         ops.rotate_kv_write(q, k, v, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, rotary, vrot,
                             ctx.positions, ctx.row_of_token, cache.k, cache.v, table, cache.page_size,
-                            write_kv=cache.write, interleaved_values=self.interleaved_values)
+                            write_kv=write, interleaved_values=self.interleaved_values)
         ops.window_attention(q, act, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, cache.k, cache.v,
                              table, cache.page_size, ctx, self.scale, self.window or 0, vrot, self.interleaved_values)
+
+
+class LatentAttention(ProjectedPart, Mixer):
+    """Softmax attention whose keys and values all come from ONE latent vector a token.
+
+    ``W_down x`` has ``latent_dim + rot_dim`` rows: the first ``latent_dim``, divided by their root
+    mean square and multiplied by a weight, are the latent ``c``; the rest are one rotated key part
+    for all heads.  Head h's key is ``[W_uk,h c, rotated part]`` against the query
+    ``[q_h unrotated (head_dim), q_h rotated (rot_dim)]``, its value ``W_uv,h c``.  The cache holds ``c``
+    and the rotated part only, as ONE key/value head with keys ``[c, rotated part]`` and values ``c``:
+    the score ``q_h . (W_uk,h c)`` is ``(W_uk,h^T q_h) . c``, so each query head is taken into the
+    latent space (``head_linear``), attention runs over the latents with all heads sharing the one
+    key/value head, and each head's weighted sum of latents goes through ``W_uv,h`` afterwards.
+
+    ``pos_enc`` turns the first ``pos_enc.rot_dim`` features of a rotated part; ``interleaved``: the
+    checkpoint pairs feature 2i with 2i + 1, so the rows that make the rotated parts are reordered
+    when they are loaded (even features, then odd ones), which leaves every score as it was.
+    Tensor names: ``q, dkv, dkv.norm, uk, uv, o`` unless given."""
+
+    is_mixer = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, latent_dim: int,
+                 scale: float, norm_eps: float, pos_enc: Optional[PositionEncoding] = None, interleaved: bool = True,
+                 names: Optional[Dict[str, str]] = None):
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.head_dim, self.rot_dim = int(num_heads), int(head_dim), int(rot_dim)
+        self.v_head_dim, self.latent_dim = int(v_head_dim), int(latent_dim)
+        self.scale, self.norm_eps = float(scale), float(norm_eps)
+        self.pos_enc, self.interleaved = pos_enc, bool(interleaved)
+        self.names = {"q": "q", "down": "dkv", "norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o"}
+        if names:
+            self.names.update(names)
+
+    def in_projections(self):
+        n = self.names
+        return [(n["q"], self.num_heads * (self.head_dim + self.rot_dim)), (n["down"], self.latent_dim + self.rot_dim)]
+
+    def out_projection(self):
+        return (self.names["o"], self.num_heads * self.v_head_dim)
+
+    def own_specs(self):
+        n, H, R = self.names, self.num_heads, self.latent_dim
+        return {n["norm"]: ParamSpec((R,), "norm"), n["uk"]: ParamSpec((H * self.head_dim, R)),
+                n["uv"]: ParamSpec((H * self.v_head_dim, R))}
+
+    def cache_need(self):
+        return PagedKVNeed(1, self.latent_dim + self.rot_dim, None, self.latent_dim)
+
+    def _pairs_apart(self, part: torch.Tensor) -> torch.Tensor:
+        """Rows of one rotated part [rot_dim, hidden] with the turned pairs' halves apart."""
+        rot = self.pos_enc.rot_dim if self.pos_enc is not None else 0
+        if not self.interleaved or rot == 0:
+            return part
+        return torch.cat([part[0:rot:2], part[1:rot:2], part[rot:]], dim=0)
+
+    def arrange_in(self, name: str, w: torch.Tensor) -> torch.Tensor:
+        d, r, R = self.head_dim, self.rot_dim, self.latent_dim
+        if name == self.names["q"]:
+            heads = w.view(self.num_heads, d + r, w.shape[1])
+            return torch.cat([torch.cat([h[:d], self._pairs_apart(h[d:])], dim=0) for h in heads], dim=0)
+        if name == self.names["down"]:
+            return torch.cat([w[:R], self._pairs_apart(w[R:])], dim=0)
+        return w
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        n, H, R = self.names, self.num_heads, self.latent_dim
+        if not rt.ops.window_attention_supported(H, 1, R + self.rot_dim, R):
+            raise ValueError(f"latent attention with {H} heads over a latent of {R} + {self.rot_dim} features is beyond "
+                             f"the window attention kernel (32 heads, 256 features)")
+        self.norm_weight = tensors[n["norm"]].to(device=rt.device, dtype=torch.float32).contiguous()
+        uk = tensors[n["uk"]].to(device=rt.device, dtype=rt.dtype)
+        self.w_absorb = uk.view(H, self.head_dim, R).transpose(1, 2).contiguous()        # [H, R, head_dim]: W_uk,h^T
+        self.w_value = tensors[n["uv"]].to(device=rt.device, dtype=rt.dtype).contiguous().view(H, self.v_head_dim, R)
+
+    def core(self, ctx, proj, act, cache) -> None:
+        ops, n, ws = self.rt.ops, self.names, ctx.workspace
+        H, d, r, R = self.num_heads, self.head_dim, self.rot_dim, self.latent_dim
+        q, down = proj[n["q"]], proj[n["down"]]
+        T = q.shape[0]
+        table = ctx.block_tables[cache.group]
+        q_lat = ws.get("latent.q", T, H * (R + r), self.rt.dtype)
+        rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
+        ops.latent_kv_write(q, down, q_lat, H, d, r, R, self.norm_weight, self.norm_eps, rotary, ctx.positions,
+                            ctx.row_of_token, cache.k, cache.v, table, cache.page_size, write_kv=cache.write)
+        ops.head_linear(q, d + r, self.w_absorb, q_lat, R + r)
+        lat = ws.get("latent.sum", T, H * R, self.rt.dtype)
+        ops.window_attention(q_lat, lat, H, 1, R + r, R, cache.k, cache.v, table, cache.page_size, ctx, self.scale, 0, None, False)
+        ops.head_linear(lat, R, self.w_value, act, self.v_head_dim)

@@ -298,6 +298,11 @@ class ProjectedPart(Part):
     def load_own(self, tensors, rt: Runtime) -> None:
         self.rt = rt
 
+    def arrange_in(self, name: str, w: torch.Tensor) -> torch.Tensor:
+        """The rows of the in-projection ``name`` in the order ``core`` wants them (a part that turns
+        pairs of neighbouring features may ask for the pairs' halves apart, say); as stored by default."""
+        return w
+
     def core(self, ctx, proj, act, cache) -> None:
         raise NotImplementedError
 
@@ -371,7 +376,7 @@ class ProjectionSet:
         for (prefix, part), views, (a0, cols) in zip(self.members, self.in_slices, self.act_slices):
             sub = narrow_tensors(tensors, prefix) if prefix else tensors
             for name, (c0, rows) in views.items():
-                w_in[c0:c0 + rows] = sub[name].to(device=rt.device, dtype=rt.dtype)
+                w_in[c0:c0 + rows] = part.arrange_in(name, sub[name].to(device=rt.device, dtype=rt.dtype))
             w_out[:, a0:a0 + cols] = sub[part.out_projection()[0]].to(device=rt.device, dtype=rt.dtype)
             if a0 > end:
                 self._gaps.append((end, a0))

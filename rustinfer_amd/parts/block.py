@@ -23,12 +23,13 @@ class Hidden:
     (``pending``) or, with ``x`` complete, the input that a sub-layer has already prepared for
     the sub-layer behind a given norm (``deferred = (that norm, DeferredNorm)``)."""
 
-    __slots__ = ("x", "pending", "deferred")
+    __slots__ = ("x", "pending", "deferred", "act")
 
     def __init__(self, x: torch.Tensor):
         self.x = x
         self.pending = None
         self.deferred = None
+        self.act = None          # x rounded to the run dtype, if a block has left it (blocks whose sub-layers read x itself)
 
     def input_behind(self, ctx, norm, out: torch.Tensor):
         """What the sub-layer behind ``norm`` reads: the prepared input if there is one for this
@@ -215,3 +216,70 @@ class ParallelBlock(Part):
         leaves in its cache or state; ``hidden`` is not meaningful afterwards."""
         if self.mixer is not None:
             self._run(ctx, hidden, cache, True)
+
+
+class PostNormBlock(Part):
+    """Sub-layers that read the residual stream itself, and a norm on what each returns:
+    ``x <- x + norm1(mixer(x)); x <- x + norm2(ffn(x))`` (the norms are ``OutputRMSNorm``: they carry
+    the factor on the branch and add to the stream themselves).  The feed-forward may be absent.
+
+    The stream is 32-bit; a sub-layer is given its rounding to the run dtype, which the norm before
+    it writes beside the stream in the same pass (``Hidden.act``); in a 32-bit run it is the stream."""
+
+    takes_follow = False
+    leaves_act = True            # forward() leaves the stream's rounding in Hidden.act
+
+    def __init__(self, hidden_size: int, mixer: Mixer, mixer_norm: Norm, ffn: Optional[FeedForward] = None,
+                 ffn_norm: Optional[Norm] = None, names: Optional[Dict[str, str]] = None):
+        if mixer is None or mixer_norm is None or (ffn is None) != (ffn_norm is None):
+            raise ValueError("a block needs a mixer, and a sub-layer and its norm come together")
+        self.hidden_size = int(hidden_size)
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+        self.names = {"mixer_norm": "norm1", "mixer": "mix", "ffn_norm": "norm2", "ffn": "mlp"}
+        if names:
+            self.names.update(names)
+
+    def _children(self):
+        for key in ("mixer_norm", "mixer", "ffn_norm", "ffn"):
+            part = getattr(self, key)
+            if part is not None:
+                yield self.names[key], part
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = {}
+        for prefix, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[join_name(prefix, name)] = spec
+        return specs
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        for prefix, part in self._children():
+            part.load(narrow_tensors(tensors, prefix), rt)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", True) for _, part in self._children())
+
+    def can_cut_rows(self) -> bool:
+        return False
+
+    def entry(self):
+        return (None, self.mixer)
+
+    def forward(self, ctx, hidden: Hidden, cache, out_rows=None, follow=None) -> None:
+        x = hidden.x
+        if hidden.pending is not None or hidden.deferred is not None:
+            raise RuntimeError("a block whose sub-layers read the stream itself needs the stream complete")
+        exact = self.rt.dtype == torch.float32
+        act = None if exact else ctx.workspace.get("block.stream_act", x.shape[0], self.hidden_size, self.rt.dtype)
+        if not exact and hidden.act is None:
+            self.rt.ops.norm_residual(x, None, None, 1.0, act=act)       # the stream's rounding, nothing added
+        inp = x if exact else act
+        self.mixer_norm.add(ctx, x, self.mixer.forward(ctx, inp, cache), act)
+        if self.ffn is not None:
+            self.ffn_norm.add(ctx, x, self.ffn.forward(ctx, inp), act)
+        hidden.act = act

@@ -15,11 +15,12 @@ from .base import ParamSpec, Part, Runtime, split_normed, stored_to
 
 
 class Embedding(Part):
-    def __init__(self, vocab_size: int, dim: int, weight_name: str = "weight"):
+    def __init__(self, vocab_size: int, dim: int, weight_name: str = "weight", scale: float = 1.0):
         self.vocab_size = int(vocab_size)
         self.dim = int(dim)
         self.weight = None
         self.weight_name = weight_name       # "" where the table carries the part's own name
+        self.scale = float(scale)            # every embedded row is multiplied by it
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {self.weight_name: ParamSpec((self.vocab_size, self.dim), "matrix")}
@@ -29,13 +30,16 @@ class Embedding(Part):
         self.weight = stored_to(tensors[self.weight_name], rt)
 
     def forward(self, ctx, ids: torch.Tensor, out_x: torch.Tensor) -> torch.Tensor:
-        self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None))
+        if self.scale != 1.0:
+            self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None), scale=self.scale)
+        else:
+            self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None))
         return out_x
 
 
 class LMHead(Part):
     def __init__(self, vocab_size: int, dim: int, tied_to: Optional[Embedding] = None,
-                 logit_scale: float = 1.0, softcap: float = 0.0):
+                 logit_scale: float = 1.0, softcap: float = 0.0, weight_name: str = "weight"):
         """``logit_scale``, ``softcap``: the logits leave as ``softcap * tanh(logit_scale * z / softcap)``
         (``softcap = 0``: ``logit_scale * z``)."""
         self.vocab_size = int(vocab_size)
@@ -43,18 +47,19 @@ class LMHead(Part):
         self.tied_to = tied_to
         self.weight = None
         self.logit_scale, self.softcap = float(logit_scale), float(softcap)
+        self.weight_name = weight_name       # "" where the matrix carries the part's own name
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         if self.tied_to is not None:
             return {}
-        return {"weight": ParamSpec((self.vocab_size, self.dim), "matrix")}
+        return {self.weight_name: ParamSpec((self.vocab_size, self.dim), "matrix")}
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         if self.tied_to is not None:
             self.weight = self.tied_to.weight      # same storage, no copy
         else:
-            self.weight = stored_to(tensors["weight"], rt)
+            self.weight = stored_to(tensors[self.weight_name], rt)
         self.weight_tiled = rt.tile(self.weight)
 
     takes_deferred_norm = True

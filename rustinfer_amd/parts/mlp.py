@@ -7,7 +7,7 @@ crates/infer-backend-cuda/src/kernels/swiglu/swiglu.cu:294-343).
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
@@ -16,26 +16,30 @@ from .linear import Linear
 
 
 class SwiGLUMLP(FeedForward):
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, names: Optional[Dict[str, str]] = None,
+                 delta_dtype: Optional[torch.dtype] = None):
+        """``names``: the tensors' names (``gate``, ``up``, ``down``) where they are not the usual
+        ``*_proj.weight``.  ``delta_dtype = torch.float32``: the down projection's 32-bit sums leave
+        unrounded (for a block that norms what the feed-forward returns)."""
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.gate_up = Linear(self.hidden_size, 2 * self.intermediate_size)
         self.down = Linear(self.intermediate_size, self.hidden_size)
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        if names:
+            self.names.update(names)
+        self.delta_dtype = delta_dtype
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        h, i = self.hidden_size, self.intermediate_size
-        return {
-            "gate_proj.weight": ParamSpec((i, h)),
-            "up_proj.weight": ParamSpec((i, h)),
-            "down_proj.weight": ParamSpec((h, i)),
-        }
+        h, i, n = self.hidden_size, self.intermediate_size, self.names
+        return {n["gate"]: ParamSpec((i, h)), n["up"]: ParamSpec((i, h)), n["down"]: ParamSpec((h, i))}
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
-        gate = tensors["gate_proj.weight"].to(device=rt.device, dtype=rt.dtype)
-        up = tensors["up_proj.weight"].to(device=rt.device, dtype=rt.dtype)
+        gate = tensors[self.names["gate"]].to(device=rt.device, dtype=rt.dtype)
+        up = tensors[self.names["up"]].to(device=rt.device, dtype=rt.dtype)
         self.gate_up.set_weight(torch.cat([gate, up], dim=0), rt)
-        self.down.set_weight(tensors["down_proj.weight"], rt)
+        self.down.set_weight(tensors[self.names["down"]], rt)
 
     takes_deferred_norm = True
 
@@ -54,7 +58,8 @@ class SwiGLUMLP(FeedForward):
 
     def forward(self, ctx, normed) -> torch.Tensor:
         act = self._activation(ctx, normed)
-        return self.rt.ops.linear_delta(act, self.down.weight, ctx.workspace, "ffn.out", self.down.weight_tiled)
+        return self.rt.ops.linear_delta(act, self.down.weight, ctx.workspace, "ffn.out", self.down.weight_tiled,
+                                        out_dtype=self.delta_dtype)
 
     def forward_into(self, ctx, normed, x: torch.Tensor, next_norm):
         """Few rows: the down projection adds its sums to ``x`` itself and prepares the input behind
@@ -94,3 +99,54 @@ class DenseMLP(ProjectedPart, FeedForward):
 
     def forward(self, ctx, normed):
         return ProjectedPart.forward(self, ctx, normed, None)
+
+
+class MoEFeedForward(FeedForward):
+    """``experts`` gated feed-forwards of width ``expert_size`` of which every token uses ``top``: the
+    router's logits ``W_router x`` and their softmax over all experts are 32-bit; the ``top`` largest
+    probabilities are the chosen experts' weights (divided by their sum only with ``renormalize``); the
+    output is the weighted sum of the chosen experts' ``W_down (silu(W_gate x) * W_up x)``.
+
+    The experts' gate and up matrices are stacked into one product for all of them, every expert's
+    activation is multiplied by its token's weight (0 where it was not chosen), and the experts' down
+    matrices side by side make the weighted sum in ONE product: three launches whatever the number of
+    experts, nothing that depends on which experts a token chose (so a step can be captured), and
+    the same arithmetic for a token whatever else is in the step.  Every token pays for all experts;
+    with few tokens in a step the experts' weights are read once either way.
+    Tensor names: ``router``, ``e<i>.gate``, ``e<i>.up``, ``e<i>.down``."""
+
+    def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, renormalize: bool = False):
+        if not (0 < top <= experts):
+            raise ValueError(f"top {top} of {experts} experts")
+        self.hidden_size, self.expert_size = int(hidden_size), int(expert_size)
+        self.experts, self.top, self.renormalize = int(experts), int(top), bool(renormalize)
+        self.router = Linear(self.hidden_size, self.experts)
+        self.gate_up = Linear(self.hidden_size, 2 * self.experts * self.expert_size)
+        self.down = Linear(self.experts * self.expert_size, self.hidden_size)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        h, f = self.hidden_size, self.expert_size
+        specs = {"router": ParamSpec((self.experts, h))}
+        for e in range(self.experts):
+            specs[f"e{e}.gate"], specs[f"e{e}.up"], specs[f"e{e}.down"] = ParamSpec((f, h)), ParamSpec((f, h)), ParamSpec((h, f))
+        return specs
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        to = lambda name: tensors[name].to(device=rt.device, dtype=rt.dtype)
+        self.router.set_weight(to("router"), rt, tile=False)
+        self.gate_up.set_weight(torch.cat([to(f"e{e}.{n}") for e in range(self.experts) for n in ("gate", "up")], dim=0), rt)
+        self.down.set_weight(torch.cat([to(f"e{e}.down") for e in range(self.experts)], dim=1), rt)
+
+    def forward(self, ctx, normed) -> torch.Tensor:
+        ops, ws = self.rt.ops, ctx.workspace
+        T, E, F = normed.shape[0], self.experts, self.expert_size
+        logits = ws.get("moe.logits", T, E, torch.float32)
+        self.router.forward(normed, logits)
+        weights = ws.get("moe.weights", T, E, torch.float32)
+        ops.moe_route(logits, weights, self.top, self.renormalize)
+        gate_up = ws.get("moe.gate_up", T, 2 * E * F, self.rt.dtype)
+        self.gate_up.forward(normed, gate_up)
+        act = ws.get("moe.act", T, E * F, self.rt.dtype)
+        ops.moe_swiglu_weighted(gate_up, weights, act, E, F)
+        return ops.linear_delta(act, self.down.weight, ws, "moe.out", self.down.weight_tiled, out_dtype=torch.float32)

@@ -17,20 +17,27 @@ from .base import Norm, ParamSpec, Runtime, stored_to
 
 
 class RMSNorm(Norm):
-    def __init__(self, dim: int, eps: float, weight_name: str = "weight"):
+    def __init__(self, dim: int, eps: float, weight_name: str = "weight", one_plus: bool = False):
         """``weight_name``: the weight's name under the norm's own ("" where the tensor carries the
-        norm's name itself)."""
+        norm's name itself).  ``one_plus``: the checkpoint stores the weight around zero and the norm
+        multiplies by ``1 + w`` (kept as that sum, in 32-bit)."""
         self.dim = int(dim)
         self.eps = float(eps)
         self.weight = None
         self.weight_name = weight_name
+        self.one_plus = bool(one_plus)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
+        if self.one_plus:
+            return {self.weight_name: ParamSpec((self.dim,), mean=0.0, std=0.1)}
         return {self.weight_name: ParamSpec((self.dim,), "norm")}
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = stored_to(tensors[self.weight_name], rt, keep_fp32=True)
+        if self.one_plus:
+            self.weight = (tensors[self.weight_name].to(device=rt.device, dtype=torch.float32) + 1.0).contiguous()
+        else:
+            self.weight = stored_to(tensors[self.weight_name], rt, keep_fp32=True)
 
     cuts_rows = True          # forward() takes x_rows (see PreNormBlock.forward)
     # nothing but ``weight`` and ``eps``: the sub-layers around this norm may do it between them
@@ -40,3 +47,29 @@ class RMSNorm(Norm):
     def forward(self, ctx, x, delta, out, rows=None, x_rows=None):
         self.rt.ops.add_rmsnorm(x, delta, self.weight, self.eps, out, rows, x_rows)
         return out
+
+
+class OutputRMSNorm(Norm):
+    """The norm of a block whose sub-layers read the residual stream itself: it sits on a sub-layer's
+    OUTPUT, and what it leaves is added to the stream, ``x += mult * y * rsqrt(mean(y^2) + eps) * w``
+    with ``w`` the stored weight, or ``1 + w`` with ``one_plus``.  All in 32-bit, the weight too."""
+
+    def __init__(self, dim: int, eps: float, mult: float = 1.0, weight_name: str = "weight", one_plus: bool = False):
+        self.dim, self.eps, self.mult = int(dim), float(eps), float(mult)
+        self.weight = None
+        self.weight_name = weight_name
+        self.one_plus = bool(one_plus)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        if self.one_plus:
+            return {self.weight_name: ParamSpec((self.dim,), mean=0.0, std=0.1)}
+        return {self.weight_name: ParamSpec((self.dim,), "norm")}
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.weight = tensors[self.weight_name].to(device=rt.device, dtype=torch.float32).contiguous()
+
+    def add(self, ctx, x, delta, act=None):
+        """``x`` (32-bit stream) gains the normed ``delta`` ([T, d], or a stack of 32-bit partial sums);
+        ``act`` takes the new rows in its dtype, for the sub-layer that reads the stream next."""
+        self.rt.ops.norm_residual(x, delta, self.weight, self.eps, mult=self.mult, one_plus=self.one_plus, act=act)

@@ -121,3 +121,49 @@ class GeneralDeltaRule(ProjectedPart, Mixer):
                         self.head_dim, self.head_dim, wl=wl, al=proj[n["a"]], w0=self.w0, ab=self.a_bias,
                         unit_eps=self.unit_eps, decay_c=self.decay_strength)
         ops.gated_group_norm(o, self.norm_weight, proj[n["g"]], act, self.head_dim, self.norm_eps)
+
+
+class Retention(ProjectedPart, Mixer):
+    """``S <- decay_h S + k v^T``, ``o = S^T q`` with one fixed decay a head, no softmax and no
+    denominator; q and k are turned by the token's position (``pos_enc``: the first ``rot_dim``
+    features, feature i with i + rot_dim/2) and k is multiplied by ``key_scale`` after that; each head's
+    ``o`` is divided by its root mean square (no weight), the heads are gated by ``silu(W_g x)`` and
+    projected.  Rotation, state and norm are 32-bit.  Tensor names: ``q, k, v, g, o`` unless given."""
+
+    is_mixer = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, decay: Sequence[float],
+                 norm_eps: float, pos_enc=None, key_scale: Optional[float] = None, names: Optional[Dict[str, str]] = None):
+        if len(decay) != num_heads:
+            raise ValueError(f"{len(decay)} decays for {num_heads} heads")
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.head_dim, self.v_head_dim = int(num_heads), int(head_dim), int(v_head_dim)
+        self.decay_values = [float(x) for x in decay]
+        self.norm_eps = float(norm_eps)
+        self.pos_enc = pos_enc
+        self.key_scale = float(key_scale) if key_scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.names = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o"}
+        if names:
+            self.names.update(names)
+
+    def in_projections(self):
+        n, hk, hv = self.names, self.num_heads * self.head_dim, self.num_heads * self.v_head_dim
+        return [(n["q"], hk), (n["k"], hk), (n["v"], hv), (n["g"], hv)]
+
+    def out_projection(self):
+        return (self.names["o"], self.num_heads * self.v_head_dim)
+
+    def cache_need(self):
+        return StateNeed((self.num_heads, self.head_dim, self.v_head_dim), torch.float32)
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=rt.device)
+
+    def core(self, ctx, proj, act, cache) -> None:
+        ops, n = self.rt.ops, self.names
+        o = ctx.workspace.get("scan.o", act.shape[0], self.num_heads * self.v_head_dim, torch.float32)
+        ops.linear_scan(proj[n["q"]], proj[n["k"]], proj[n["v"]], cache.state, o, ctx, self.num_heads, self.head_dim,
+                        self.v_head_dim, decay=self.decay, rotary=self.pos_enc.rotary() if self.pos_enc is not None else None,
+                        k_scale=self.key_scale)
+        ops.gated_group_norm(o, None, proj[n["g"]], act, self.v_head_dim, self.norm_eps, gate_activation="silu")

@@ -4,16 +4,17 @@ from __future__ import annotations
 
 from typing import Callable, Dict
 
-from .attention import PagedAttention, WindowAttention
-from .mlp import DenseMLP, SwiGLUMLP
-from .norm import RMSNorm
-from .recurrent import GeneralDeltaRule, LightningAttention
+from .attention import LatentAttention, PagedAttention, WindowAttention
+from .mlp import DenseMLP, MoEFeedForward, SwiGLUMLP
+from .norm import OutputRMSNorm, RMSNorm
+from .recurrent import GeneralDeltaRule, LightningAttention, Retention
 from .rope import RotaryEmbedding
 
 MIXERS: Dict[str, Callable] = {"attention": PagedAttention, "window_attention": WindowAttention,
-                               "lightning": LightningAttention, "general_delta": GeneralDeltaRule}
-FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP, "dense": DenseMLP}
-NORMS: Dict[str, Callable] = {"rmsnorm": RMSNorm}
+                               "lightning": LightningAttention, "general_delta": GeneralDeltaRule,
+                               "latent_attention": LatentAttention, "retention": Retention}
+FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP, "dense": DenseMLP, "moe": MoEFeedForward}
+NORMS: Dict[str, Callable] = {"rmsnorm": RMSNorm, "output_rmsnorm": OutputRMSNorm}
 POSITION_ENCODINGS: Dict[str, Callable] = {"rope": RotaryEmbedding}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,

@@ -1,4 +1,4 @@
-"""Rotary position encoding with the llama3 frequency rescale.
+"""Rotary position encoding with the llama3 frequency rescale, or YaRN's.
 
 Frequencies ``f_i = theta^(-2i/rot_dim)``; llama3 scaling keeps wavelengths
 shorter than ``O/high``, divides those longer than ``O/low`` by ``factor`` and
@@ -16,14 +16,22 @@ from typing import Optional
 
 import torch
 
-from ..config.model_config import RopeScaling
+from ..config.model_config import RopeScaling, YarnScaling
 from .base import PositionEncoding, Runtime
 
 
 def rotary_frequencies(rot_dim: int, theta: float, scaling: Optional[RopeScaling]) -> torch.Tensor:
     half = rot_dim // 2
     freqs = [1.0 / (theta ** (2.0 * i / rot_dim)) for i in range(half)]
-    if scaling is not None:
+    if isinstance(scaling, YarnScaling):
+        # the pair index at which a frequency makes `turns` turns over the original length
+        at = lambda turns: rot_dim * math.log(scaling.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+        lo = max(math.floor(at(scaling.fast)), 0)
+        hi = min(math.ceil(at(scaling.slow)), rot_dim - 1)
+        for i, f in enumerate(freqs):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            freqs[i] = f / scaling.factor * ramp + f * (1.0 - ramp)
+    elif scaling is not None:
         orig = float(scaling.original_max_position_embeddings)
         lam_low = orig / scaling.low_freq_factor
         lam_high = orig / scaling.high_freq_factor
@@ -41,8 +49,8 @@ def rotary_frequencies(rot_dim: int, theta: float, scaling: Optional[RopeScaling
 
 
 class RotaryEmbedding(PositionEncoding):
-    def __init__(self, head_dim: int, theta: float, scaling: Optional[RopeScaling] = None,
-                 rot_dim: Optional[int] = None):
+    def __init__(self, head_dim: int, theta: float, scaling=None, rot_dim: Optional[int] = None):
+        """``scaling``: None, a ``RopeScaling`` (llama3) or a ``YarnScaling``."""
         self.head_dim = int(head_dim)
         self.rot_dim = int(rot_dim if rot_dim is not None else head_dim)
         if self.rot_dim % 2 or not (0 < self.rot_dim <= self.head_dim):
@@ -59,8 +67,10 @@ class RotaryEmbedding(PositionEncoding):
         freqs = rotary_frequencies(self.rot_dim, self.theta, self.scaling)
         pos = torch.arange(max_positions, dtype=torch.float64)
         ang = pos[:, None] * freqs[None, :]
-        self.cos = ang.cos().to(torch.float32).to(rt.device).contiguous()
-        self.sin = ang.sin().to(torch.float32).to(rt.device).contiguous()
+        # a stretched rotation also lengthens the vectors it turns (YarnScaling)
+        mag = 0.1 * math.log(self.scaling.factor) + 1.0 if isinstance(self.scaling, YarnScaling) else 1.0
+        self.cos = (ang.cos() * mag).to(torch.float32).to(rt.device).contiguous()
+        self.sin = (ang.sin() * mag).to(torch.float32).to(rt.device).contiguous()
         self.max_positions = max_positions
 
     def rotary(self):
