@@ -348,7 +348,7 @@ class TedelixBench(Bench):
         from rustinfer_amd.llm import LLM
         self.torch, self.args = torch, args
         self.window = 1024
-        conf = tedelix_config(shape_name, args.layers, self.window)
+        conf = self.design_config(shape_name, args)
         self.full_layers = SHAPES[shape_name]["num_hidden_layers"]
         self.prompt_len = args.context // 2
         self.dir = tempfile.TemporaryDirectory()
@@ -371,6 +371,13 @@ class TedelixBench(Bench):
                 n *= int(d)
             self.params += n
         self.weight_bytes = el * self.params
+        self.gen = torch.Generator(device="cuda").manual_seed(1)
+        self.account(cfg, el)
+
+    def design_config(self, shape_name, args):
+        return tedelix_config(shape_name, args.layers, self.window)
+
+    def account(self, cfg, el):
         # what a decoding request reads a step beside the weights: the keys and values inside its
         # windows, and its states (read and written back, 32-bit)
         self.window_kv_bytes = self.state_bytes = 0
@@ -386,7 +393,6 @@ class TedelixBench(Bench):
             else:
                 self.state_bytes += 2 * 4 * m.heads * m.dim * m.dim
                 self.scan_flops_per_token += 2.0 * 5 * m.heads * m.dim * m.dim
-        self.gen = torch.Generator(device="cuda").manual_seed(1)
 
     @property
     def kv_bytes_per_token(self):          # Bench.decode prices a step as weights + batch * context * this
@@ -415,17 +421,80 @@ class TedelixBench(Bench):
                 "product_flops": products, "mixer_flops_32bit": mixers}
 
 
+# Belorax at the layer sizes of the Llama shapes: the same width, number of layers and heads; its
+# mixers take turns (every fourth layer reads the keys and values of the attention layer three before
+# it); the latent is as wide as the attention kernels take beside a rotated part of half a head; gated
+# feed-forwards of the shape's width alternate with eight experts of a quarter of it, two a token
+# (the same weights in all, half of them used by a token).
+BELORAX_PATTERN = ("attention", "latent_attention", "retention", "attention")
+
+
+def belorax_config(shape_name, layers=0):
+    s = SHAPES[shape_name]
+    H, G, hd, W, ff = s["num_attention_heads"], s["num_key_value_heads"], s["head_dim"], s["hidden_size"], s["intermediate_size"]
+    out = []
+    for i in range(layers or s["num_hidden_layers"]):
+        kind = BELORAX_PATTERN[i % len(BELORAX_PATTERN)]
+        if kind == "attention":
+            mixer = dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, q_temp=dict(coef=0.1, every=1024))
+            if i % len(BELORAX_PATTERN) == 3:
+                mixer["kv_from"] = i - 3
+        elif kind == "latent_attention":
+            r = hd // 2
+            mixer = dict(heads=H, dim=hd, rot_dim=r, vdim=hd, kv_rank=256 - r, scale=(hd + r) ** -0.5,
+                         rot=dict(base=10000.0, dims=r, scaling=dict(factor=4.0, original=4096, fast=32.0, slow=1.0)))
+        else:
+            mixer = dict(heads=H, dim=hd, vdim=hd, decay=[1.0 - 2.0 ** (-5 - 3 * h / max(H - 1, 1)) for h in range(H)],
+                         rot=dict(base=10000.0, dims=hd))
+        mlp = dict(kind="dense", ff=ff) if i % 2 == 0 else dict(kind="moe", expert=dict(ff=ff // 4), router=dict(experts=8, top=2))
+        out.append(dict(type=kind, mixer=mixer, mlp=mlp))
+    return dict(architecture="Belorax", vocab=s["vocab_size"], width=W, norm=dict(eps=1e-6), embedding=dict(scale=1.0),
+                residual_mult=0.5, layers=out)
+
+
+class BeloraxBench(TedelixBench):
+    """The same measurements on a Belorax model of a Llama shape's sizes."""
+
+    def design_config(self, shape_name, args):
+        self.window = 1 << 30                         # no window: a request reads all its keys
+        return belorax_config(shape_name, args.layers)
+
+    def account(self, cfg, el):
+        self.window_kv_bytes = self.state_bytes = 0
+        self.attn_flops_per_key = self.scan_flops_per_token = 0
+        for layer in cfg.layers:
+            m = layer.mixer
+            if layer.type == "attention":
+                self.window_kv_bytes += m.kv_heads * (m.dim + m.vdim) * el          # a borrowed cache is read again
+                self.attn_flops_per_key += 2.0 * m.heads * (m.dim + m.vdim)
+            elif layer.type == "latent_attention":
+                self.window_kv_bytes += (2 * m.kv_rank + m.rot_dim) * el            # the latent lies there as key and as value
+                self.attn_flops_per_key += 2.0 * m.heads * (2 * m.kv_rank + m.rot_dim)
+                self.scan_flops_per_token += 2.0 * m.heads * m.kv_rank * (m.dim + m.vdim)      # into the latent space and back
+            else:
+                self.state_bytes += 2 * 4 * m.heads * m.dim * m.vdim
+                self.scan_flops_per_token += 2.0 * 2 * m.heads * m.dim * m.vdim
+
+
+DESIGNS = {"tedelix": (TedelixBench, "llama", TEDELIX_PATTERN), "belorax": (BeloraxBench, "tedelix", BELORAX_PATTERN)}
+
+
 def design_record(args, peaks):
-    """``--design tedelix``: decode at the main batch and prefill of 2,048 tokens for Tedelix models of
-    the sizes of ``--design-shapes``, each beside the Llama model of the same sizes."""
-    out = {"metric": "decode tok/s at batch %d and prefill tok/s at 2,048 tokens: Tedelix beside Llama at equal layer sizes" % args.batch,
+    """``--design tedelix|belorax``: decode at the main batch and prefill of 2,048 tokens for models of
+    that design at the sizes of ``--design-shapes``, each beside the closest other design at the same
+    sizes (Tedelix beside Llama, Belorax beside Tedelix)."""
+    cls, beside, pattern = DESIGNS[args.design]
+    others = {"llama": Bench, "tedelix": TedelixBench}
+    out = {"metric": "decode tok/s at batch %d and prefill tok/s at 2,048 tokens: %s beside %s at equal layer sizes" % (args.batch, args.design, beside),
            "unit": "tok/s", "dtype": args.dtype, "data": "synthetic: random weights, random token ids", "peaks": peaks,
-           "pattern": list(TEDELIX_PATTERN), "window": 1024, "shapes": {}}
+           "pattern": list(pattern), "shapes": {}}
+    if args.design == "tedelix":
+        out["window"] = 1024
     steps = max(MIN_POINT_STEPS, args.steps)
     for name in args.design_shapes.split(","):
         rec = {}
-        for who, cls in (("tedelix", TedelixBench), ("llama", Bench)):
-            if who == "llama" and args.no_points:
+        for who, cls in ((args.design, cls), (beside, others[beside])):
+            if who == beside and args.no_points:
                 continue
             b = cls(name, args, args.batch)
             tok_s, step_s, step_bytes = b.decode(args.batch, steps, args.warmup)
@@ -516,10 +585,11 @@ def main() -> int:
                     help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",
                     help="keep the GEMM library's own choice of kernel for the prompt's products")
-    ap.add_argument("--design", default="llama", choices=["llama", "tedelix"],
-                    help="tedelix: only decode and prefill of Tedelix models at the sizes of --design-shapes, each beside "
-                         "the Llama model of the same sizes (the default workload is not run)")
-    ap.add_argument("--design-shapes", default="1b,3b", help="shapes for --design tedelix, with commas between them")
+    ap.add_argument("--design", default="llama", choices=["llama", "tedelix", "belorax"],
+                    help="tedelix, belorax: only decode and prefill of models of that design at the sizes of --design-shapes, "
+                         "each beside the closest other design at the same sizes (Tedelix beside Llama, Belorax beside "
+                         "Tedelix; the default workload is not run)")
+    ap.add_argument("--design-shapes", default="1b,3b", help="shapes for --design tedelix|belorax, with commas between them")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -530,7 +600,7 @@ def main() -> int:
         print(json.dumps(sampling_times(ops, SHAPES[args.shape]["vocab_size"], args.steps)))
         return 0
     peaks = ops.measure_peaks()
-    if args.design == "tedelix":
+    if args.design in DESIGNS:
         print(json.dumps(design_record(args, peaks)))
         return 0
     b = Bench(args.shape, args, max(args.batch, 16 if args.mixed else 1 if (args.no_points or args.prompt) else 64))

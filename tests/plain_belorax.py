@@ -135,9 +135,10 @@ def qknorm_attention(h, w, m, eps, kv):
     T, H, G = h.shape[0], m["heads"], m["kv_heads"]
     k, v = kv
     q = unit((h @ w["q"].T).reshape(T, H, m["dim"]), eps) * w["q.norm"]
-    p = np.arange(T)
-    temp = 1.0 + m["q_temp"]["coef"] * np.log(np.floor((p + 1) / m["q_temp"]["every"]) + 1.0)
-    q = q * temp[:, None, None]
+    if m.get("q_temp"):
+        p = np.arange(T)
+        temp = 1.0 + m["q_temp"]["coef"] * np.log(np.floor((p + 1) / m["q_temp"]["every"]) + 1.0)
+        q = q * temp[:, None, None]
     heads = [causal_softmax_attention(q[:, i], k[:, i // (H // G)], v[:, i // (H // G)], m["scale"]) for i in range(H)]
     return np.concatenate(heads, axis=1) @ w["o"].T
 
@@ -189,9 +190,14 @@ def gated_ff(h, w):
     return (silu(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T
 
 
-def routed_ff(h, w, mlp):
+def routed_ff(h, w, mlp, gaps=None):
+    """``gaps`` (a list) receives, for every row, how far the last chosen expert's probability lies
+    above the first one left out, relative to it (infinite where all experts are chosen)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     s = softmax_rows(h @ w["router"].T)
+    if gaps is not None:
+        ranked = -np.sort(-s, axis=1)
+        gaps.append((ranked[:, top - 1] - ranked[:, top]) / ranked[:, top - 1] if top < E else np.full(h.shape[0], np.inf))
     out = np.zeros((h.shape[0], w["e0.down"].shape[0]))
     for t in range(h.shape[0]):
         for e in np.argsort(-s[t], kind="stable")[:top]:
@@ -206,9 +212,10 @@ def _sub(w: Dict[str, np.ndarray], prefix: str) -> Dict[str, np.ndarray]:
     return {k[len(prefix):]: a for k, a in w.items() if k.startswith(prefix)}
 
 
-def forward(cfg: dict, w: Dict[str, np.ndarray], ids, layers_out: Optional[List[np.ndarray]] = None) -> np.ndarray:
+def forward(cfg: dict, w: Dict[str, np.ndarray], ids, layers_out: Optional[List[np.ndarray]] = None,
+            gaps: Optional[List[np.ndarray]] = None) -> np.ndarray:
     """Logits [T, vocab] of one sequence from its first token.  ``layers_out`` collects the
-    residual stream after every layer."""
+    residual stream after every layer, ``gaps`` every routed layer's margins (``routed_ff``)."""
     eps, mult = cfg["norm"]["eps"], cfg["residual_mult"]
     x = w["embed"][np.asarray(ids, dtype=np.int64)] * cfg["embedding"]["scale"]
     kept = {}
@@ -228,7 +235,7 @@ def forward(cfg: dict, w: Dict[str, np.ndarray], ids, layers_out: Optional[List[
         mlp = layer.get("mlp")
         if mlp is not None:
             fw = _sub(w, f"l{i}.mlp.")
-            y = gated_ff(x, fw) if mlp["kind"] == "dense" else routed_ff(x, fw, mlp)
+            y = gated_ff(x, fw) if mlp["kind"] == "dense" else routed_ff(x, fw, mlp, gaps)
             x = x + mult * unit(y, eps) * (1.0 + w[f"l{i}.norm2"])
         if layers_out is not None:
             layers_out.append(x.copy())

@@ -1,0 +1,150 @@
+"""Belorax without a GPU: the configuration reader, the tensors the model asks for, its run order
+with borrowed caches, the cache manager's books for its layers, and the stretched rotary frequencies."""
+import math
+
+import numpy as np
+import pytest
+
+import plain_belorax as P
+from rustinfer_amd.config import BeloraxConfig, ConfigError, resolve_architecture
+from rustinfer_amd.config.model_config import (FeedForwardSpec, LatentAttentionSpec, NormedAttentionSpec, RetentionSpec,
+                                               YarnScaling)
+
+CFG = dict(architecture="Belorax", vocab=97, width=48, norm=dict(eps=3e-6), embedding=dict(scale=2.5), residual_mult=0.25, layers=[
+    dict(type="attention", mixer=dict(heads=6, kv_heads=2, dim=8, vdim=12, scale=0.3, q_temp=dict(coef=0.7, every=9)), mlp=dict(kind="dense", ff=56)),
+    dict(type="retention", mixer=dict(heads=2, dim=16, vdim=8, decay=[0.9, 0.99], rot=dict(base=777.0, dims=6)), mlp=None),
+    dict(type="latent_attention", mixer=dict(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=20, scale=0.2,
+                                              rot=dict(base=5000.0, dims=6, scaling=dict(factor=3.0, original=128, fast=16.0, slow=2.0))),
+         mlp=dict(kind="moe", expert=dict(ff=24), router=dict(experts=5, top=2))),
+    dict(type="attention", mixer=dict(heads=2, kv_heads=2, dim=8, vdim=12, scale=0.4, kv_from=0), mlp=dict(kind="dense", ff=8)),
+])
+
+
+def changed(path, value):
+    import copy
+    d = copy.deepcopy(CFG)
+    node = d
+    for k in path[:-1]:
+        node = node[k]
+    if value is KeyError:
+        del node[path[-1]]
+    else:
+        node[path[-1]] = value
+    return d
+
+
+def test_reads_every_size_and_constant():
+    entry = resolve_architecture(CFG)
+    assert entry.name == "Belorax"
+    c = BeloraxConfig.from_dict(CFG)
+    assert (c.vocab_size, c.hidden_size, c.norm_eps, c.embedding_scale, c.residual_mult) == (97, 48, 3e-6, 2.5, 0.25)
+    a, r, l, b = (x.mixer for x in c.layers)
+    assert a == NormedAttentionSpec(6, 2, 8, 12, 0.3, 0.7, 9, None)
+    assert r == RetentionSpec(2, 16, 8, (0.9, 0.99), 777.0, 6)
+    assert l == LatentAttentionSpec(3, 10, 6, 14, 20, 0.2, 5000.0, 6, YarnScaling(3.0, 128, 16.0, 2.0))
+    assert b == NormedAttentionSpec(2, 2, 8, 12, 0.4, 0.0, 0, 0)
+    assert [x.mlp for x in c.layers] == [FeedForwardSpec("dense", 56), None, FeedForwardSpec("moe", 24, 5, 2), FeedForwardSpec("dense", 8)]
+    assert BeloraxConfig.from_dict(c.to_dict()) == c
+
+
+@pytest.mark.parametrize("change,word", [
+    ((("layers", 0, "type"), "conv"), "unknown mixer"), ((("layers", 0, "mixer", "kv_heads"), 4), "multiple"),
+    ((("layers", 3, "mixer", "kv_from"), 1), "kv_from"), ((("layers", 3, "mixer", "kv_from"), 3), "kv_from"),
+    ((("layers", 3, "mixer", "vdim"), 16), "equal"), ((("layers", 1, "mixer", "decay"), [0.5]), "decay"),
+    ((("layers", 1, "mixer", "rot", "dims"), 18), "rot.dims"), ((("layers", 2, "mixer", "rot", "dims"), 8), "rot.dims"),
+    ((("layers", 2, "mlp", "router", "top"), 6), "top"), ((("layers", 2, "mlp", "kind"), "sparse"), "kind"),
+    ((("layers", 2, "mixer", "rot", "scaling", "factor"), KeyError), "factor"), ((("width",), KeyError), "width"),
+    ((("layers", 0, "mixer", "q_temp", "every"), 0), "every"), ((("norm", "eps"), 0.0), "eps")])
+def test_refuses_what_it_cannot_run(change, word):
+    with pytest.raises(ConfigError) as e:
+        BeloraxConfig.from_dict(changed(*change))
+    assert word in str(e.value)
+
+
+def build():
+    entry = resolve_architecture(CFG)
+    return entry.builder(BeloraxConfig.from_dict(CFG))
+
+
+def test_model_asks_for_the_designs_tensors():
+    W = 48
+    want = {"embed": (97, W), "head": (97, W), "final.norm": (W,)}
+    for i in range(4):
+        want[f"l{i}.norm1"] = (W,)
+    want.update({"l0.norm2": (W,), "l2.norm2": (W,), "l3.norm2": (W,)})
+    want.update({"l0.mix.q": (48, W), "l0.mix.k": (16, W), "l0.mix.v": (24, W), "l0.mix.q.norm": (8,), "l0.mix.k.norm": (8,), "l0.mix.o": (W, 72),
+                 "l0.mlp.gate": (56, W), "l0.mlp.up": (56, W), "l0.mlp.down": (W, 56)})
+    want.update({"l1.mix.q": (32, W), "l1.mix.k": (32, W), "l1.mix.v": (16, W), "l1.mix.g": (16, W), "l1.mix.o": (W, 16)})
+    want.update({"l2.mix.q": (48, W), "l2.mix.dkv": (26, W), "l2.mix.dkv.norm": (20,), "l2.mix.uk": (30, 20), "l2.mix.uv": (42, 20),
+                 "l2.mix.o": (W, 42), "l2.mlp.router": (5, W)})
+    for e in range(5):
+        want.update({f"l2.mlp.e{e}.gate": (24, W), f"l2.mlp.e{e}.up": (24, W), f"l2.mlp.e{e}.down": (W, 24)})
+    want.update({"l3.mix.q": (16, W), "l3.mix.q.norm": (8,), "l3.mix.o": (W, 24),
+                 "l3.mlp.gate": (8, W), "l3.mlp.up": (8, W), "l3.mlp.down": (W, 8)})
+    got = {n: tuple(s.shape) for n, s in build().param_specs().items()}
+    assert got == want
+
+
+def test_run_order_and_cache_needs_with_a_borrowed_cache():
+    from rustinfer_amd.parts.base import PagedKVNeed, StateNeed
+    import torch
+    model = build()
+    assert [(c.layer, c.cache, c.write) for c in model.schedule] == [(0, 0, True), (1, 1, True), (2, 2, True), (3, 0, False)]
+    needs = model.cache_needs()
+    assert needs == {0: PagedKVNeed(2, 8, None, 12), 1: StateNeed((2, 16, 8), torch.float32), 2: PagedKVNeed(1, 26, None, 20)}
+
+
+def test_cache_books_for_these_layers():
+    from rustinfer_amd.cache import CacheManager
+    cm = CacheManager(build().cache_needs(), page_size=16, num_pages=6, max_requests=2, max_model_len=96)
+    assert len(cm.groups) == 2 and 1 not in [cid for g in cm.groups for cid in g.cache_ids]
+    cm.add_request("a")
+    cm.append("a", 40)
+    cm.add_request("b")
+    cm.append("b", 17)
+    assert not cm.can_append([("a", 30)]) and cm.can_append([("a", 8)])      # five of six pages are out
+    assert not cm.can_append([("c", 1)])                                      # and both state slots
+    held = set(cm.table(0, "a"))
+    cm.release("a")
+    cm.add_request("c")
+    cm.append("c", 48)
+    assert set(cm.table(0, "c")) & held                                       # pages are used again
+    cm.check()
+
+
+@pytest.mark.parametrize("dims,base,sc", [(16, 1e6, dict(factor=2.0, original=1024, fast=32.0, slow=1.0)),
+                                          (64, 1e4, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
+                                          (2, 10.0, dict(factor=4.0, original=64, fast=8.0, slow=2.0)),
+                                          (6, 5000.0, dict(factor=3.0, original=128, fast=16.0, slow=2.0))])
+def test_stretched_frequencies(dims, base, sc):
+    from rustinfer_amd.parts import rotary_frequencies
+    got = rotary_frequencies(dims, base, YarnScaling(**sc)).numpy()
+    want, mag = P.yarn_frequencies(dims, base, sc)
+    assert np.allclose(got, want, rtol=1e-13, atol=0)
+    assert mag == 0.1 * math.log(sc["factor"]) + 1.0
+    plain = P.plain_frequencies(dims, base)
+    assert np.all(got <= plain * (1 + 1e-12)) and np.all(got >= plain / sc["factor"] * (1 - 1e-12))
+
+
+def test_plain_mechanisms_reduce_to_known_cases():
+    """The oracle itself: one expert of weight one is the gated feed-forward; retention without decay
+    and rotation is a running sum of outer products; a latent layer's score is the dot product of the
+    expanded keys; the interleaved and the halves rotation agree up to the order of features."""
+    rng = np.random.default_rng(0)
+    h = rng.standard_normal((7, 10))
+    w = {"router": rng.standard_normal((1, 10)), "e0.gate": rng.standard_normal((6, 10)), "e0.up": rng.standard_normal((6, 10)),
+         "e0.down": rng.standard_normal((10, 6))}
+    assert np.allclose(P.routed_ff(h, w, dict(router=dict(experts=1, top=1))), P.gated_ff(h, P._sub(w, "e0.")))
+    y = rng.standard_normal((5, 8))
+    f = P.plain_frequencies(8, 100.0)
+    perm = np.concatenate([np.arange(0, 8, 2), np.arange(1, 8, 2)])
+    assert np.allclose(P.rotate(y, f, 8, True)[:, perm], P.rotate(y[:, perm], f, 8, False))
+    assert np.allclose(np.linalg.norm(P.rotate(y, f, 8, True, 1.3), axis=1), 1.3 * np.linalg.norm(y, axis=1))
+    m = dict(heads=1, dim=4, vdim=3, decay=[1.0], rot=dict(base=10.0, dims=2))
+    eye = np.eye(4)
+    wr = {"q": eye, "k": eye, "v": rng.standard_normal((3, 4)), "g": rng.standard_normal((3, 4)), "o": np.eye(3)}
+    x = rng.standard_normal((6, 4))
+    x[:, :2] = 0.0                                           # nothing in the rotated features
+    out = P.retention(x, wr, m, 1e-9)
+    o = np.stack([sum((x[t] @ x[j]) / 2.0 * (wr["v"] @ x[j]) for j in range(t + 1)) for t in range(6)])
+    assert np.allclose(out, P.unit(o, 1e-9) * P.silu(x @ wr["g"].T))

@@ -1,0 +1,621 @@
+"""Belorax on the GPU against the plain implementation (``plain_belorax.py``): every mechanism
+alone, then whole models of three small configurations that differ in every size and in the order
+of their layers, through every way of cutting requests into steps, through pages and state slots
+that are used again, and through ``LLM.generate``.  Weights are drawn here with deviations that
+make activations of order one, and a few tests build inputs so that one far key decides."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_belorax as P
+from helpers import cut_mixed, cut_portions, cut_tail_single, cut_whole, random_requests, run_steps
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+YARN = dict(factor=4.0, original=64, fast=8.0, slow=2.0)
+
+
+def att(heads, kv, dim, vdim, scale, coef=0.0, every=0, kv_from=None):
+    m = dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale)
+    if every:
+        m["q_temp"] = dict(coef=coef, every=every)
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return dict(type="attention", mixer=m)
+
+
+def lat(heads, dim, rot_dim, vdim, rank, scale, base=10000.0, dims=None, scaling=None):
+    rot = dict(base=base, dims=dims or rot_dim)
+    if scaling:
+        rot["scaling"] = scaling
+    return dict(type="latent_attention", mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=rank, scale=scale, rot=rot))
+
+
+def ret(heads, dim, vdim, decay, base=10000.0, dims=None):
+    return dict(type="retention", mixer=dict(heads=heads, dim=dim, vdim=vdim, decay=decay, rot=dict(base=base, dims=dims or dim)))
+
+
+def dense(ff):
+    return dict(kind="dense", ff=ff)
+
+
+def moe(experts, top, ff):
+    return dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top))
+
+
+def layer(mixer, mlp):
+    return dict(mixer, mlp=mlp)
+
+
+CONFIGS = {
+    # a borrowed cache two layers on, one expert a token, a layer without feed-forward, a temperature that moves every 5
+    "A": dict(architecture="Belorax", vocab=200, width=64, norm=dict(eps=1e-5), embedding=dict(scale=1.7), residual_mult=0.8, layers=[
+        layer(ret(2, 16, 8, [0.9, 0.6], base=100.0, dims=8), moe(4, 1, 24)),
+        layer(att(4, 2, 16, 24, 0.3, coef=0.4, every=5), dense(96)),
+        layer(lat(3, 8, 4, 12, 20, 0.35, base=50.0), None),
+        layer(att(4, 2, 16, 24, 0.25, coef=1.0, every=16, kv_from=1), moe(6, 6, 8)),
+        layer(lat(2, 24, 8, 8, 16, 0.2, base=1000.0, scaling=YARN), dense(40)),
+    ]),
+    # heads beyond one 64-wide slice, a latent beyond 128, more experts than a wave has lanes, two borrowers of one cache
+    "B": dict(architecture="Belorax", vocab=333, width=136, norm=dict(eps=1e-6), embedding=dict(scale=1.0), residual_mult=1.0, layers=[
+        layer(att(8, 2, 72, 132, 0.11), moe(70, 3, 16)),
+        layer(lat(5, 40, 16, 72, 136, 0.1, base=200.0, dims=12, scaling=dict(factor=2.0, original=32, fast=4.0, slow=1.0)), dense(200)),
+        layer(att(4, 2, 72, 132, 0.12, coef=0.3, every=64, kv_from=0), None),
+        layer(ret(3, 72, 40, [0.999, 0.8, 0.3], base=50000.0), dense(64)),
+        layer(att(2, 2, 72, 132, 0.09, coef=2.0, every=3, kv_from=0), dense(136)),
+        layer(ret(1, 128, 130, [0.97], base=300.0, dims=64), moe(3, 2, 40)),
+    ]),
+    # a width and a vocabulary that are no multiples of eight, three and six query heads a key/value head, one head
+    "C": dict(architecture="Belorax", vocab=211, width=100, norm=dict(eps=1e-6), embedding=dict(scale=0.5), residual_mult=0.3, layers=[
+        layer(lat(1, 12, 6, 10, 9, 0.4, base=20.0, dims=2), moe(5, 2, 12)),
+        layer(att(3, 1, 24, 40, 0.2, coef=0.7, every=2), dense(50)),
+        layer(ret(5, 20, 12, [0.9, 0.8, 0.7, 0.6, 0.5], base=10.0, dims=20), dense(30)),
+        layer(att(12, 2, 16, 18, 0.25), None),
+        layer(lat(6, 10, 10, 14, 40, 0.3, base=500.0, scaling=dict(factor=8.0, original=16, fast=2.0, slow=0.5)), dense(77)),
+    ]),
+}
+PAGE = {"A": 8, "B": 16, "C": 16}
+
+
+def bf16_round(a: np.ndarray) -> torch.Tensor:
+    return torch.tensor(a, dtype=torch.float32).to(torch.bfloat16)
+
+
+def draw_weights(cfg: dict, seed: int):
+    """name -> bfloat16 tensor for every tensor of the design, activations of order one."""
+    rng = np.random.default_rng(seed)
+    W = cfg["width"]
+    mat = lambda o, i, s=1.0: bf16_round(s * rng.standard_normal((o, i)) / math.sqrt(i))
+    vec = lambda n, mean, std: bf16_round(mean + std * rng.standard_normal(n))
+    t = {"embed": bf16_round(rng.standard_normal((cfg["vocab"], W))), "final.norm": vec(W, 0.0, 0.1), "head": mat(cfg["vocab"], W)}
+    for i, lay in enumerate(cfg["layers"]):
+        m, p = lay["mixer"], f"l{i}."
+        t[p + "norm1"] = vec(W, 0.0, 0.1)
+        if lay["type"] == "attention":
+            t[p + "mix.q"], t[p + "mix.q.norm"] = mat(m["heads"] * m["dim"], W), vec(m["dim"], 1.0, 0.2)
+            if m.get("kv_from") is None:
+                t[p + "mix.k"], t[p + "mix.k.norm"] = mat(m["kv_heads"] * m["dim"], W), vec(m["dim"], 1.0, 0.2)
+                t[p + "mix.v"] = mat(m["kv_heads"] * m["vdim"], W)
+            t[p + "mix.o"] = mat(W, m["heads"] * m["vdim"])
+        elif lay["type"] == "latent_attention":
+            H, d, r, R = m["heads"], m["dim"], m["rot_dim"], m["kv_rank"]
+            t[p + "mix.q"], t[p + "mix.dkv"], t[p + "mix.dkv.norm"] = mat(H * (d + r), W, 2.0), mat(R + r, W, 2.0), vec(R, 1.0, 0.2)
+            t[p + "mix.uk"], t[p + "mix.uv"], t[p + "mix.o"] = mat(H * d, R, 2.0), mat(H * m["vdim"], R), mat(W, H * m["vdim"])
+        else:
+            hk, hv = m["heads"] * m["dim"], m["heads"] * m["vdim"]
+            t[p + "mix.q"], t[p + "mix.k"], t[p + "mix.v"], t[p + "mix.g"] = mat(hk, W), mat(hk, W), mat(hv, W), mat(hv, W)
+            t[p + "mix.o"] = mat(W, hv)
+        mlp = lay["mlp"]
+        if mlp is not None:
+            t[p + "norm2"] = vec(W, 0.0, 0.1)
+            if mlp["kind"] == "dense":
+                t[p + "mlp.gate"], t[p + "mlp.up"], t[p + "mlp.down"] = mat(mlp["ff"], W), mat(mlp["ff"], W), mat(W, mlp["ff"])
+            else:
+                F = mlp["expert"]["ff"]
+                t[p + "mlp.router"] = mat(mlp["router"]["experts"], W, 3.0)
+                for e in range(mlp["router"]["experts"]):
+                    t[p + f"mlp.e{e}.gate"], t[p + f"mlp.e{e}.up"], t[p + f"mlp.e{e}.down"] = mat(F, W), mat(F, W), mat(W, F)
+    return t
+
+
+@pytest.fixture(scope="module")
+def tdirs(tmp_path_factory):
+    from rustinfer_amd.weights import write_safetensors
+    out = {}
+    for k, (name, cfg) in enumerate(CONFIGS.items()):
+        d = str(tmp_path_factory.mktemp("belorax_" + name))
+        with open(os.path.join(d, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        write_safetensors(os.path.join(d, "model.safetensors"), draw_weights(cfg, 31 + k))
+        out[name] = d
+    return out
+
+
+@pytest.fixture(scope="module")
+def plain(tdirs):
+    return {name: P.read_model(d) for name, d in tdirs.items()}
+
+
+@pytest.fixture(scope="module")
+def plain_logits(plain):
+    memo = {}
+
+    def get(name, lengths, seed):
+        key = (name, tuple(lengths), seed)
+        if key not in memo:
+            cfg, w = plain[name]
+            reqs = random_requests(cfg["vocab"], lengths, seed)
+            memo[key] = (reqs, plain_rows(cfg, w, reqs))
+        return memo[key]
+    return get
+
+
+class Rows(dict):
+    """request -> plain logits [T, vocab]; ``margin[request][t]``: the smallest margin by which a router
+    chose its experts for token t (over the routed layers)."""
+    margin = None
+
+
+def plain_rows(cfg, w, reqs):
+    rows = Rows()
+    rows.margin = {}
+    for rid, toks in reqs.items():
+        gaps = []
+        rows[rid] = P.forward(cfg, w, toks, gaps=gaps)
+        rows.margin[rid] = np.min(np.stack(gaps), axis=0) if gaps else np.full(len(toks), np.inf)
+    return rows
+
+
+def engine_for(model_dir, dtype, name, num_pages=64, max_requests=4, max_len=512):
+    from rustinfer_amd.engine import build_engine
+    return build_engine(model_dir, dtype=dtype, device=DEV, page_size=PAGE[name], num_pages=num_pages,
+                        max_requests=max_requests, max_model_len=max_len, max_batch_tokens=2048)
+
+
+# a row of logits: root mean square of the difference (its mean taken off) over the deviation of
+# the plain logits.  32-bit rounds at 1e-7, and every row must be within 2e-4: that is the sharp
+# test, and the bfloat16 run goes through the same kernels.  bfloat16 rounds at 4e-3 a time, and this
+# design passes that on more than most: every sub-layer's output is brought to unit size before it is
+# added, sharp softmaxes turn a rounded score into another weight, and a token whose router's last
+# chosen expert lies within a few hundredths of the first one left out goes to that one (0.3 at that
+# row, and the rows that attend to it inherit some of it).  Measured on these weights, the median row
+# lies at 1e-2 (A) to 5e-2 (B, six layers at residual_mult 1), one row in five over 6e-2.  A wrong
+# key, a lost state or a wrong expert for every token gives 0.3 to 1 at every row behind it.  So in
+# bfloat16 the median row must be within 8e-2, nine in ten within 0.25 and every one within 1; rows of
+# tokens with such a close call (the plain implementation says which) are not judged.
+TOL = {"float32": 2e-4}
+CLOSE_CALL = 0.05
+
+
+def check_rows(steps, results, logits, dtype, label):
+    s = max(float(np.std(v)) for v in logits.values())
+    pos, errs = {}, []
+    most = 1.0 if dtype == "bfloat16" else TOL[dtype]
+    margin = getattr(logits, "margin", None) if dtype == "bfloat16" else None
+    for st in steps:
+        got, row = results.get(st["step"]), 0
+        for e in st["entries"]:
+            p0 = pos.get(e["id"], 0)
+            for w in e["want"]:
+                d = got[row].astype(np.float64) - logits[e["id"]][p0 + w]
+                err = float(np.sqrt(np.mean((d - d.mean()) ** 2))) / s
+                row += 1
+                if margin is not None and margin[e["id"]][p0 + w] < CLOSE_CALL:
+                    continue
+                assert err <= most, (f"{label}: step {st['step']} request {e['id']} position {p0 + w} (place {w} of a "
+                                     f"portion of {len(e['tokens'])} from {p0}): row error {err:.2e} of the deviation")
+                errs.append(err)
+            pos[e["id"]] = p0 + len(e["tokens"])
+        for rid in st["end"]:
+            pos.pop(rid, None)
+    if dtype == "bfloat16":
+        over = sum(e > 0.25 for e in errs)
+        assert over * 10 <= len(errs), f"{label}: {over} of {len(errs)} rows are over 0.25"
+        assert float(np.median(errs)) <= 8e-2, f"{label}: the median row error is {np.median(errs):.2e}"
+    return max(errs)
+
+
+# ---------------------------------------------------------------------------
+# each mechanism alone
+# ---------------------------------------------------------------------------
+class OnePart:
+    """The least a 'model' must be for the engine to build a step context around one mixer."""
+    vocab_size = 100
+
+    def __init__(self, mixer, pos_encs=()):
+        self.mixer, self.pos_encs = mixer, list(pos_encs)
+
+    def prepare(self, rt, max_positions):
+        for pe in self.pos_encs:
+            pe.prepare(rt, max_positions)
+
+    def cache_needs(self):
+        need = self.mixer.cache_need()
+        return {0: need} if need is not None else {}
+
+
+def run_part(part, pos_encs, dtype, x, cuts, page=8, batch_with=None):
+    """The part's output [T, hidden] for one sequence ``x [T, hidden]`` fed in portions of ``cuts``.
+    ``batch_with``: rows of a second request that shares every step (its output is dropped)."""
+    from rustinfer_amd.engine import Engine, StepEntry, make_runtime
+    rt = make_runtime(dtype, DEV)
+    eng = Engine(OnePart(part, pos_encs), rt, page_size=page, num_pages=160, max_requests=3, max_model_len=640)
+    outs, pos, other = [], 0, 0
+    for n in cuts:
+        entries, rows = [StepEntry("a", [0] * n, [])], [x[pos:pos + n]]
+        if batch_with is not None and other < batch_with.shape[0]:
+            m = min(3, batch_with.shape[0] - other)
+            entries.insert(0, StepEntry("b", [0] * m, []))
+            rows.insert(0, batch_with[other:other + m])
+            other += m
+        starts = []
+        for e in entries:
+            if not eng.cache.has_request(e.request_id):
+                eng.cache.add_request(e.request_id)
+            starts.append(eng.cache.append(e.request_id, len(e.tokens)))
+        ctx = eng._build_context(entries, starts)
+        inp = torch.cat(rows).to(DEV, rt.dtype).contiguous()
+        cache = eng.cache.view(0) if 0 in eng.cache else None
+        out = part.forward(ctx, inp, cache) if getattr(part, "is_mixer", False) else part.forward(ctx, inp)
+        out = out.double().sum(0) if out.dim() == 3 else out.double()
+        outs.append(out[-n:].cpu().numpy())
+        pos += n
+    return np.concatenate(outs)
+
+
+def part_weights(part, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    wt = {}
+    for n, s in part.param_specs().items():
+        if len(s.shape) == 2:
+            wt[n] = (torch.randn(s.shape, generator=g) * scale / math.sqrt(s.shape[1])).to(torch.bfloat16)
+        else:
+            wt[n] = (1.0 + torch.randn(s.shape, generator=g) * 0.2).to(torch.bfloat16)
+    return wt, {n: t.double().numpy() for n, t in wt.items()}
+
+
+def rel(a, b):
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-9))
+
+
+PART_TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+CUTS = (13, 1, 1, 2, 30, 1, 7, 2, 1, 1, 1, 1, 40, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 5)
+
+
+def some_rows(T, d, seed):
+    return torch.randn(T, d, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16).float()
+
+
+@pytest.fixture(params=["matrix", "fma"])
+def portion_kernel(request):
+    """Steps with prompt portions on the matrix-instruction kernel (the default) and on the FMA one."""
+    from rustinfer_amd.kernels import ops
+    keep, ops.WINDOW_ATTENTION_MFMA = ops.WINDOW_ATTENTION_MFMA, request.param == "matrix"
+    yield request.param
+    ops.WINDOW_ATTENTION_MFMA = keep
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,dk,dv,scale,coef,every", [
+    (4, 2, 16, 24, 0.3, 0.5, 4), (3, 3, 40, 36, 0.2, 0.0, 0), (8, 1, 32, 16, 0.18, 2.0, 1), (2, 2, 128, 128, 0.09, 0.3, 64),
+    (5, 5, 72, 200, 0.12, 0.9, 7), (6, 1, 24, 40, 0.2, 1.5, 30), (2, 1, 256, 256, 0.06, 0.1, 2), (1, 1, 6, 2, 0.5, 0.5, 3)])
+def test_normed_attention_alone(dtype, H, G, dk, dv, scale, coef, every, portion_kernel):
+    from rustinfer_amd.engine import make_runtime
+    from rustinfer_amd.parts import WindowAttention
+    d = 48
+    part = WindowAttention(d, H, G, dk, dv, scale, qk_norm_eps=1e-5, q_temperature=(coef, every) if every else None)
+    wt, w = part_weights(part, H * dk + every, scale=2.0)
+    part.load(wt, make_runtime(dtype, DEV))
+    x = some_rows(sum(CUTS), d, 5)
+    m = dict(heads=H, kv_heads=G, dim=dk, vdim=dv, scale=scale, q_temp=dict(coef=coef, every=every or 1 << 30))
+    xs = x.double().numpy()
+    ref = P.qknorm_attention(xs, w, m, 1e-5, P.attention_keys_values(xs, w, m, 1e-5))
+    assert rel(run_part(part, [], dtype, x, CUTS), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,d,r,dv,R,dims,scaling", [
+    (3, 8, 4, 12, 20, 4, None), (8, 32, 16, 32, 64, 16, dict(factor=2.0, original=64, fast=16.0, slow=1.0)),
+    (1, 12, 6, 10, 9, 2, YARN), (5, 40, 16, 72, 136, 12, YARN), (16, 16, 8, 24, 48, 8, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
+    (2, 64, 64, 130, 192, 64, YARN), (32, 4, 2, 4, 6, 2, None)])
+def test_latent_attention_alone(dtype, H, d, r, dv, R, dims, scaling, portion_kernel):
+    from rustinfer_amd.config import YarnScaling
+    from rustinfer_amd.engine import make_runtime
+    from rustinfer_amd.parts import LatentAttention, RotaryEmbedding
+    width = 56
+    pe = RotaryEmbedding(r, 300.0, scaling=YarnScaling(**scaling) if scaling else None, rot_dim=dims)
+    part = LatentAttention(width, H, d, r, dv, R, 0.3 / math.sqrt(d + r), 1e-5, pos_enc=pe)
+    wt, w = part_weights(part, H * d + R, scale=2.0)
+    part.load(wt, make_runtime(dtype, DEV))
+    x = some_rows(sum(CUTS), width, 6)
+    rot = dict(base=300.0, dims=dims)
+    if scaling:
+        rot["scaling"] = scaling
+    m = dict(heads=H, dim=d, rot_dim=r, vdim=dv, kv_rank=R, scale=0.3 / math.sqrt(d + r), rot=rot)
+    ref = P.latent_attention(x.double().numpy(), w, m, 1e-5)
+    assert rel(run_part(part, [pe], dtype, x, CUTS), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,dk,dv,decay,dims", [(2, 16, 24, [0.9, 0.5], 16), (3, 72, 40, [0.999, 0.7, 0.2], 36), (1, 128, 64, [0.95], 2),
+                                                (4, 64, 64, [0.98, 0.99, 0.997, 0.9995], 64), (1, 256, 8, [0.9], 128), (2, 20, 130, [1.0, 0.0], 20)])
+def test_retention_alone(dtype, H, dk, dv, decay, dims):
+    from rustinfer_amd.engine import make_runtime
+    from rustinfer_amd.parts import Retention, RotaryEmbedding
+    width = 40
+    pe = RotaryEmbedding(dk, 100.0, rot_dim=dims)
+    part = Retention(width, H, dk, dv, decay, 1e-5, pos_enc=pe)
+    wt, w = part_weights(part, H * dk + dv, scale=2.0)
+    part.load(wt, make_runtime(dtype, DEV))
+    x = some_rows(sum(CUTS), width, 7)
+    other = some_rows(60, width, 8)
+    m = dict(heads=H, dim=dk, vdim=dv, decay=decay, rot=dict(base=100.0, dims=dims))
+    ref = P.retention(x.double().numpy(), w, m, 1e-5)
+    assert rel(run_part(part, [pe], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [pe], dtype, x, CUTS, batch_with=other), ref) < PART_TOL[dtype]     # a second request's state beside it
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("E,top,F,rows", [(4, 1, 24, 70), (16, 4, 64, 5), (70, 3, 16, 100), (6, 6, 8, 33), (3, 2, 40, 1), (130, 8, 4, 17)])
+def test_feed_forwards_alone(dtype, E, top, F, rows):
+    from types import SimpleNamespace
+    from rustinfer_amd.engine import Workspace, make_runtime
+    from rustinfer_amd.parts import MoEFeedForward, SwiGLUMLP
+    rt = make_runtime(dtype, DEV)
+    width = 40
+    x = some_rows(rows, width, 3)
+    ctx = SimpleNamespace(workspace=Workspace(rt.device))
+    part = MoEFeedForward(width, F, E, top)
+    wt, w = part_weights(part, E + top, scale=1.0)
+    wt["router"] = (wt["router"].float() * 4.0).to(torch.bfloat16)        # probabilities far apart: no close calls
+    w["router"] = wt["router"].double().numpy()
+    part.load(wt, rt)
+    out = part.forward(ctx, x.to(DEV, rt.dtype))
+    out = out.double().sum(0) if out.dim() == 3 else out.double()
+    ref = P.routed_ff(x.double().numpy(), w, dict(router=dict(experts=E, top=top)))
+    assert rel(out.cpu().numpy(), ref) < PART_TOL[dtype]
+    gated = SwiGLUMLP(width, F + 3, names={"gate": "gate", "up": "up", "down": "down"}, delta_dtype=torch.float32)
+    wt, w = part_weights(gated, 9)
+    gated.load(wt, rt)
+    out = gated.forward(ctx, x.to(DEV, rt.dtype))
+    out = out.double().sum(0) if out.dim() == 3 else out.double()
+    assert rel(out.cpu().numpy(), P.gated_ff(x.double().numpy(), w)) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width,parts", [(64, 1), (100, 3), (4096 + 8, 2), (33, 1)])
+def test_the_norm_on_a_sublayers_output(dtype, width, parts):
+    from rustinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(width)
+    T = 9
+    x = torch.randn(T, width, generator=g)
+    delta = torch.randn(parts, T, width, generator=g) * 3.0
+    wgt = (torch.randn(width, generator=g) * 0.2).to(torch.bfloat16).float()
+    d_in = delta if parts > 1 else (delta[0] if dtype == "float32" else delta[0].to(torch.bfloat16))
+    y = d_in.double().sum(0) if parts > 1 else d_in.double()
+    ref = x.double() + 0.6 * (y / torch.sqrt((y * y).mean(-1, keepdim=True) + 1e-5)) * (1.0 + wgt.double())
+    xd = x.to(DEV).contiguous()
+    act = torch.empty(T, width, device=DEV, dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    ops.norm_residual(xd, d_in.to(DEV).contiguous(), wgt.to(DEV), 1e-5, mult=0.6, one_plus=True, act=act)
+    assert rel(xd.double().cpu().numpy(), ref.numpy()) < 2e-6
+    assert rel(act.double().cpu().numpy(), ref.numpy()) < (1e-2 if dtype == "bfloat16" else 2e-6)
+
+
+def test_yarn_tables_against_the_plain_frequencies():
+    from rustinfer_amd.config import YarnScaling
+    from rustinfer_amd.engine import make_runtime
+    from rustinfer_amd.parts import RotaryEmbedding
+    for dims, base, sc in ((16, 1e6, dict(factor=2.0, original=1024, fast=32.0, slow=1.0)), (64, 1e4, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
+                           (2, 10.0, YARN), (12, 200.0, dict(factor=2.0, original=32, fast=4.0, slow=1.0))):
+        pe = RotaryEmbedding(dims, base, scaling=YarnScaling(**sc))
+        pe.prepare(make_runtime("float32", DEV), 300)
+        f, mag = P.yarn_frequencies(dims, base, sc)
+        ang = np.arange(300)[:, None] * f[None, :]
+        assert np.abs(pe.cos.cpu().numpy() - np.cos(ang) * mag).max() < 1e-6
+        assert np.abs(pe.sin.cpu().numpy() - np.sin(ang) * mag).max() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("decoded", [False, True])
+@pytest.mark.parametrize("kind", ["normed", "latent"])
+def test_one_far_key_decides(dtype, decoded, kind, portion_kernel):
+    """A query that matches one key hundreds of positions back, in the first page's first slot, in
+    a page's last slot and just behind a page border: the output is that key's value.  Were the key
+    lost (a wrong page, a wrong table entry, a block of keys left out) the output would be a mean
+    of all values instead."""
+    from rustinfer_amd.engine import make_runtime
+    from rustinfer_amd.parts import LatentAttention, RotaryEmbedding, WindowAttention
+    T, dk, dv = 420, 16, 12
+    g = torch.Generator().manual_seed(2)
+    eye = torch.eye(dk)
+    look = torch.zeros(dk, dk)                              # a query reads feature 8 + n into key feature n
+    marked = {0: 300, 15: 340, 16: 380, 271: 419}          # key position -> the query that looks for it
+    x = 0.1 * torch.randn(T, dk, generator=g)
+    x[:, 8:] = 0.0
+    x[:, 14] = 3.0                                          # keeps the other keys' few features small after the norm
+    for n, (kpos, qpos) in enumerate(marked.items()):
+        look[n, 8 + n] = 1.0
+        x[kpos] = 0.0
+        x[kpos, n] = 4.0
+        x[qpos, 8 + n] = 4.0
+    x = x.to(torch.bfloat16).float()
+    xs = x.double().numpy()
+    if kind == "normed":
+        part, pes = WindowAttention(dk, 1, 1, dk, dv, 2.0, qk_norm_eps=1e-6), []
+        wt = {"q": look, "k": eye, "q.norm": torch.ones(dk), "k.norm": torch.ones(dk), "v": torch.randn(dv, dk, generator=g),
+              "o": torch.randn(dk, dv, generator=g)}
+        m = dict(heads=1, kv_heads=1, dim=dk, vdim=dv, scale=2.0, q_temp=dict(coef=0.0, every=1))
+    else:
+        pe = RotaryEmbedding(2, 100.0)
+        part, pes = LatentAttention(dk, 1, dk, 2, dv, dk, 2.0, 1e-6, pos_enc=pe), [pe]
+        wt = {"q": torch.cat([look, torch.zeros(2, dk)]), "dkv": torch.cat([eye, torch.zeros(2, dk)]), "dkv.norm": torch.ones(dk),
+              "uk": eye, "uv": torch.randn(dv, dk, generator=g), "o": torch.randn(dk, dv, generator=g)}
+        m = dict(heads=1, dim=dk, rot_dim=2, vdim=dv, kv_rank=dk, scale=2.0, rot=dict(base=100.0, dims=2))
+    wt = {n: t.to(torch.bfloat16) for n, t in wt.items()}
+    part.load(wt, make_runtime(dtype, DEV))
+    w = {n: t.double().numpy() for n, t in wt.items()}
+    ref = P.qknorm_attention(xs, w, m, 1e-6, P.attention_keys_values(xs, w, m, 1e-6)) if kind == "normed" else P.latent_attention(xs, w, m, 1e-6)
+    plain_fn = (lambda z: P.qknorm_attention(z, w, m, 1e-6, P.attention_keys_values(z, w, m, 1e-6))) if kind == "normed" \
+        else (lambda z: P.latent_attention(z, w, m, 1e-6))
+    without = xs.copy()
+    without[list(marked)] = xs[1]                           # the same sequence with the marked keys gone
+    lost = plain_fn(without)
+    for qpos in marked.values():
+        assert np.abs(ref[qpos] - lost[qpos]).max() > 0.2 * np.abs(ref[qpos]).max()    # the test can tell
+    cuts = [290] + [1] * 130 if decoded else [290, 17, 50, 2, 61]
+    got = run_part(part, pes, dtype, x, cuts, page=16)
+    for qpos in marked.values():
+        assert rel(got[qpos], ref[qpos]) < PART_TOL[dtype], qpos
+
+
+# ---------------------------------------------------------------------------
+# whole models through the engine's step function
+# ---------------------------------------------------------------------------
+LENGTHS = (70, 3, 121, 1, 38)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_cut_gives_the_plain_logits(tdirs, plain_logits, name, dtype):
+    reqs, logits = plain_logits(name, LENGTHS, 21)
+    eng = engine_for(tdirs[name], dtype, name)
+    for label, steps in (("whole", cut_whole(reqs)), ("last tokens alone", cut_tail_single(reqs, tail=50)),
+                         ("portions", cut_portions(reqs, seed=3)),
+                         ("portions of two", cut_portions(reqs, seed=4, sizes=(2, 2, 3, 2, 1, 2)))):
+        check_rows(steps, run_steps(eng, steps), logits, dtype, f"{name} {dtype} {label}")
+        assert not eng.cache.live_requests()
+
+
+def test_the_stream_after_every_layer(tdirs, plain):
+    """The residual stream after each layer against the plain one: names the first layer that differs."""
+    from rustinfer_amd.engine import StepEntry
+    for name in CONFIGS:
+        cfg, w = plain[name]
+        toks = random_requests(cfg["vocab"], (45,), 9)["r0"]
+        want = []
+        P.forward(cfg, w, toks, want)
+        eng = engine_for(tdirs[name], "float32", name)
+        got = []
+        for lay in eng.model.layers:
+            def fwd(ctx, hidden, cache, _f=lay.forward, **kw):
+                _f(ctx, hidden, cache, **kw)
+                got.append(hidden.x.detach().double().cpu().numpy().copy())
+            lay.forward = fwd
+        eng.step([StepEntry("r0", toks, [0])])
+        assert len(got) == len(want)
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert rel(a, b) < 2e-5, (name, i, cfg["layers"][i]["type"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_batches_with_pages_and_slots_used_again(tdirs, plain_logits, name, dtype):
+    lengths = (90, 17, 64, 5, 130, 33, 2, 71)
+    reqs, logits = plain_logits(name, lengths, 22)
+    page = PAGE[name]
+    max_tokens = 3 * (-(-130 // 64) * 64)
+    eng = engine_for(tdirs[name], dtype, name, num_pages=max_tokens // page, max_requests=3, max_len=256)
+    steps = cut_mixed(reqs, max_tokens, seed=5, max_live=3, tail=6)
+    assert max(len(st["entries"]) for st in steps) == 3
+    slots, users = set(), {}
+    results = {}
+    from rustinfer_amd.engine import StepEntry
+    for st in steps:
+        lg = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+        slots.update(eng.cache.slot(e["id"]) for e in st["entries"])
+        for e in st["entries"]:
+            for p in eng.cache.table(0, e["id"]):
+                users.setdefault(p, set()).add(e["id"])
+        if lg.shape[0]:
+            results[st["step"]] = lg.cpu().numpy()
+        for rid in st["end"]:
+            eng.release(rid)
+    assert len(slots) == 3 and len(reqs) > 3             # eight requests went through three state slots
+    assert any(len(u) > 1 for u in users.values())       # and pages were used again
+    check_rows(steps, results, logits, dtype, f"{name} {dtype} mixed")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_a_batch_gives_what_each_request_gives_alone(tdirs, name):
+    from rustinfer_amd.engine import StepEntry
+    cfg = CONFIGS[name]
+    reqs = random_requests(cfg["vocab"], (40, 9, 1, 25), 30)
+    eng = engine_for(tdirs[name], "float32", name)
+    alone = {}
+    for rid, toks in reqs.items():
+        if len(toks) > 1:
+            eng.step([StepEntry(rid, toks[:-1], [])])
+        alone[rid] = eng.step([StepEntry(rid, toks[-1:], [0])]).cpu().numpy()[0]
+        eng.release(rid)
+    first = [StepEntry(rid, toks[:-1], []) for rid, toks in reqs.items() if len(toks) > 1]
+    eng.step(first)
+    both = eng.step([StepEntry(rid, toks[-1:], [0]) for rid, toks in reqs.items()]).cpu().numpy()
+    s = float(np.std(both))
+    for row, rid in enumerate(reqs):
+        assert np.abs(both[row] - alone[rid]).max() < 1e-4 * s, rid
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding(tdirs, plain, name):
+    """Twenty tokens of prompt and 280 single tokens: the temperature moves many times, pages fill
+    and follow one another, the state is carried 280 times."""
+    cfg, w = plain[name]
+    toks = random_requests(cfg["vocab"], (300,), 40)["r0"]
+    logits = plain_rows(cfg, w, {"r0": toks})
+    eng = engine_for(tdirs[name], "float32", name, num_pages=40)
+    steps = cut_tail_single({"r0": toks}, tail=280)
+    check_rows(steps, run_steps(eng, steps), logits, "float32", f"{name} long decoding")
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_greedy_generation_through_the_scheduler(tdirs, plain, name):
+    from rustinfer_amd.llm import LLM
+    from rustinfer_amd.sampling import SamplingParams
+    cfg, w = plain[name]
+    prompts = list(random_requests(cfg["vocab"], (12, 47, 5, 30, 21), 50).values())
+    llm = LLM(model=tdirs[name], dtype="float32", paged_block_size=PAGE[name], num_blocks=48, max_batch_seqs=3,
+              max_model_len=128, max_batch_tokens=64, chunked_prefill_size=32)
+    res = llm.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    for p, r in zip(prompts, res):
+        assert len(r.token_ids) == 12
+        toks = list(p)
+        for i, t in enumerate(r.token_ids):
+            row = P.forward(cfg, w, toks)[-1]
+            assert row.max() - row[t] < 1e-3 * max(1.0, float(np.std(row))), (i, t, int(np.argmax(row)))
+            toks.append(t)
+    assert llm.engine.graph_replays > 0 or not llm.engine._graph_sizes
+
+
+def test_trace_replay_of_a_belorax_model(tdirs, plain_logits, tmp_path):
+    """bin/trace_run as a user starts it, on the mixed cut, four state slots."""
+    import subprocess
+    import sys
+    from helpers import ROOT
+    name = "A"
+    reqs, logits = plain_logits(name, (50, 20, 9, 77, 30), 60)
+    steps = cut_mixed(reqs, 512, seed=1, max_live=4, tail=5)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", tdirs[name], "--dtype", "bfloat16",
+           "--out", str(tmp_path), "--max-tokens", "512"]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for st in steps:
+            proc.stdin.write(json.dumps(st) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {st['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=120) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    results = {}
+    for st in steps:
+        n = sum(len(e["want"]) for e in st["entries"])
+        if n:
+            results[st["step"]] = np.fromfile(os.path.join(str(tmp_path), f"{st['step']}.f32"), dtype="<f4").reshape(n, -1)
+    check_rows(steps, results, logits, "bfloat16", "trace replay")
