@@ -417,9 +417,13 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
         const T* __restrict__ q, int q_stride, const T* __restrict__ kc, const T* __restrict__ vc,
         const int* __restrict__ table, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ q_start,
         const int* __restrict__ kv_lens, int H, int Hkv, int dk, int dv, int page, float scale, int window, int slots,
-        float* __restrict__ part_ml, float* __restrict__ part_o) {
+        float* __restrict__ part_ml, float* __restrict__ part_o, int heads_a_wave) {
     extern __shared__ __align__(16) float lds[];       // [4 waves][G][64] weights
-    const int b = blockIdx.z, g = blockIdx.y, G = H / Hkv;
+    // many query heads a key/value head (one shared latent, say): the heads are dealt to several
+    // blocks in stretches of heads_a_wave, each reading the block of keys for its own heads
+    const int G = H / Hkv, stretches = (G + heads_a_wave - 1) / heads_a_wave;
+    const int b = blockIdx.z, g = blockIdx.y / stretches;
+    const int h_lo = (blockIdx.y % stretches) * heads_a_wave, h_hi = min(G, h_lo + heads_a_wave);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = cu_q[b];
     if (cu_q[b + 1] - t <= 0) return;                  // a row without a token
@@ -443,7 +447,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
     const T* qrow = q + (size_t)t * q_stride + (size_t)g * G * dk;
     const size_t at0 = ((size_t)t * H + (size_t)g * G) * slots + slot;      // + head * slots
     const bool kvec = dk % VL == 0;
-    for (int h0 = 0; h0 < G; h0 += 4) {
+    for (int h0 = h_lo; h0 < h_hi; h0 += 4) {
         float s[4] = {0.f, 0.f, 0.f, 0.f};
         if (kvec) {
             for (int dd = 0; dd < dk; dd += VL) {
@@ -453,7 +457,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
                 if (kr) ld_vec16(kr + dd, kf);
 #pragma unroll
                 for (int rb = 0; rb < 4; ++rb) {
-                    if (h0 + rb >= G) break;
+                    if (h0 + rb >= h_hi) break;
                     float qf[VL];
                     ld_vec16(qrow + (size_t)(h0 + rb) * dk + dd, qf);
 #pragma unroll
@@ -465,12 +469,12 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
                 const float kf = kr ? ld_f32(kr + dd) : 0.f;
 #pragma unroll
                 for (int rb = 0; rb < 4; ++rb)
-                    if (h0 + rb < G) s[rb] = fmaf(ld_f32(qrow + (size_t)(h0 + rb) * dk + dd), kf, s[rb]);
+                    if (h0 + rb < h_hi) s[rb] = fmaf(ld_f32(qrow + (size_t)(h0 + rb) * dk + dd), kf, s[rb]);
             }
         }
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb) {
-            if (h0 + rb >= G) break;
+            if (h0 + rb >= h_hi) break;
             float m_b, l_b;
             Ps[(h0 + rb) * AD_KEYS + lane] = aw_block_scores(s[rb], mine, scale, m_b, l_b);
             if (lane == 0) {
@@ -482,7 +486,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
     }
     __builtin_amdgcn_wave_barrier();                   // the wave's own weights are in LDS (LDS keeps a wave's order)
     const bool vvec = page % VL == 0;
-    for (int h0 = 0; h0 < G; h0 += 4) {
+    for (int h0 = h_lo; h0 < h_hi; h0 += 4) {
         float acc[4][NC];
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb)
@@ -526,7 +530,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
             }
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
-                if (h0 + rb >= G) break;
+                if (h0 + rb >= h_hi) break;
 #pragma unroll
                 for (int u = 0; u < VL; ++u) {
                     const float pv = Ps[(h0 + rb) * AD_KEYS + jj + u];
@@ -537,7 +541,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
         }
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb) {
-            if (h0 + rb >= G) break;
+            if (h0 + rb >= h_hi) break;
             float* dst = part_o + (at0 + (size_t)(h0 + rb) * slots) * dv;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
@@ -629,8 +633,13 @@ int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, con
         float* part_o = workspace + (size_t)Tn * H * slots * 2;
         auto part = NC == 1 ? attn_window_decode_kernel<T, 1> : NC == 2 ? attn_window_decode_kernel<T, 2>
                   : NC == 3 ? attn_window_decode_kernel<T, 3> : attn_window_decode_kernel<T, 4>;
-        part<<<dim3((slots + 3) / 4, Hkv, num_rows), 256, sizeof(float) * 4 * G * AD_KEYS, stream>>>(
-            q, q_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, dk, dv, page, scale, window, slots, part_ml, part_o);
+        // up to eight heads a wave: a step of few rows then still has waves for the chip's SIMDs, and
+        // a wave reads its block of keys twice at most
+        const int heads_a_wave = G <= 8 ? G : 8, stretches = (G + heads_a_wave - 1) / heads_a_wave;
+        RI_REQUIRE((long)Hkv * stretches <= 65535, "ri_attention_window: too many heads for the grid");
+        part<<<dim3((slots + 3) / 4, Hkv * stretches, num_rows), 256, sizeof(float) * 4 * G * AD_KEYS, stream>>>(
+            q, q_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, dk, dv, page, scale, window, slots, part_ml, part_o,
+            heads_a_wave);
         auto combine = NC == 1 ? attn_window_combine_kernel<T, 1> : NC == 2 ? attn_window_combine_kernel<T, 2>
                      : NC == 3 ? attn_window_combine_kernel<T, 3> : attn_window_combine_kernel<T, 4>;
         combine<<<dim3(H, num_rows), 64, 0, stream>>>(part_ml, part_o, out, out_stride, cu_q, q_start, kv_lens, H, dv, window, AD_KEYS, slots,
