@@ -483,7 +483,7 @@ def design_record(args, peaks):
     """``--design tedelix|belorax``: decode at the main batch and prefill of 2,048 tokens for models of
     that design at the sizes of ``--design-shapes``, each beside the closest other design at the same
     sizes (Tedelix beside Llama, Belorax beside Tedelix)."""
-    cls, beside, pattern = DESIGNS[args.design]
+    design_cls, beside, pattern = DESIGNS[args.design]
     others = {"llama": Bench, "tedelix": TedelixBench}
     out = {"metric": "decode tok/s at batch %d and prefill tok/s at 2,048 tokens: %s beside %s at equal layer sizes" % (args.batch, args.design, beside),
            "unit": "tok/s", "dtype": args.dtype, "data": "synthetic: random weights, random token ids", "peaks": peaks,
@@ -493,7 +493,7 @@ def design_record(args, peaks):
     steps = max(MIN_POINT_STEPS, args.steps)
     for name in args.design_shapes.split(","):
         rec = {}
-        for who, cls in ((args.design, cls), (beside, others[beside])):
+        for who, cls in ((args.design, design_cls), (beside, others[beside])):
             if who == beside and args.no_points:
                 continue
             b = cls(name, args, args.batch)

@@ -577,6 +577,7 @@ class RetentionSpec:
     decay: tuple
     rot_base: float
     rot_dims: int
+    rot_scaling: Optional[YarnScaling] = None
     kind: str = "retention"
 
     @staticmethod
@@ -585,11 +586,10 @@ class RetentionSpec:
         if not isinstance(decay, list):
             raise ConfigError(f"{where}: 'decay' must be a list with one number for each head")
         base, dims, scaling = _rot_of(m, where)
-        if scaling is not None:
-            raise ConfigError(f"{where}.rot: this mixer's rotation takes no scaling")
         s = RetentionSpec(heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where),
                           vdim=_require(m, "vdim", int, where),
-                          decay=tuple(_typed(x, "decay", float, where) for x in decay), rot_base=base, rot_dims=dims)
+                          decay=tuple(_typed(x, "decay", float, where) for x in decay), rot_base=base, rot_dims=dims,
+                          rot_scaling=scaling)
         if min(s.heads, s.dim, s.vdim) <= 0 or len(s.decay) != s.heads:
             raise ConfigError(f"{where}: heads, dim, vdim must be > 0 and 'decay' hold {s.heads} numbers")
         if s.dim > MAX_HEAD_DIM or s.rot_dims > s.dim:
@@ -599,7 +599,7 @@ class RetentionSpec:
 
     def to_dict(self) -> Dict[str, Any]:
         return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "decay": list(self.decay),
-                "rot": _rot_dict(self.rot_base, self.rot_dims)}
+                "rot": _rot_dict(self.rot_base, self.rot_dims, self.rot_scaling)}
 
 
 BELORAX_MIXERS = {"attention": NormedAttentionSpec, "latent_attention": LatentAttentionSpec, "retention": RetentionSpec}

@@ -21,7 +21,8 @@
 namespace {
 
 // ---------------------------------------------------------------------------
-// One block a token, one wave a head at a time (queries first, then keys).
+// Blocks (token, four heads): one wave a head (queries first, then keys); the blocks of a token's
+// first heads also copy its values.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_kv_write_kernel(
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(256) void head_norm_kv_write_kernel(
     const int slot = pos % page;
     const float temp = temp_every > 0 ? 1.f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.f) : 1.f;
     const int units = H + (blk >= 0 ? Hkv : 0);
-    for (int u = wave; u < units; u += 4) {
+    for (int u = blockIdx.y * 4 + wave; u < units; u += 4 * gridDim.y) {
         const bool is_q = u < H;
         const int g = u - H;
         const T* src = is_q ? q + (size_t)t * q_stride + u * dk : k + (size_t)t * k_stride + g * dk;
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(256) void head_norm_kv_write_kernel(
     }
     if (blk < 0) return;
     const T* vrow = v + (size_t)t * v_stride;
-    for (int idx = threadIdx.x; idx < Hkv * dv; idx += 256) {
+    for (int idx = blockIdx.y * 256 + threadIdx.x; idx < Hkv * dv; idx += 256 * gridDim.y) {
         const int g = idx / dv, dd = idx - g * dv;
         vc[(((size_t)blk * Hkv + g) * dv + dd) * page + slot] = vrow[idx];
     }
@@ -167,6 +168,58 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
     }
 }
 
+// The same product for a step of few tokens (up to HLF_T): no staging.  Eight lanes share an output
+// and divide K between them in pieces of 16 bytes (VEC: operands aligned for that; else element by
+// element), each summing all tokens' terms of its pieces; a block owns 32 outputs of one head.  The
+// sums of a token are added in a fixed order whatever else the step holds.
+constexpr int HLF_T = 16;
+
+__device__ __forceinline__ void hl_ld16(const float* p, float* f) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+__device__ __forceinline__ void hl_ld16(const bf16_t* p, float* f) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+    f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+    f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void head_linear_few_kernel(
+        const T* __restrict__ x, int x_stride, int x_head, const T* __restrict__ w, T* __restrict__ out, int out_stride,
+        int out_head, int Tn, int N, int K) {
+    constexpr int VL = VEC ? 16 / (int)sizeof(T) : 1;
+    const int h = blockIdx.y, part = threadIdx.x & 7, n = blockIdx.x * 32 + (threadIdx.x >> 3);
+    const bool live = n < N;
+    const T* wr = w + ((size_t)h * N + (live ? n : 0)) * K;
+    const T* xh = x + (size_t)h * x_head;
+    float acc[HLF_T];
+#pragma unroll
+    for (int t = 0; t < HLF_T; ++t) acc[t] = 0.f;
+    for (int k = part * VL; k < K; k += 8 * VL) {
+        float wv[VL];
+        if (VEC) hl_ld16(wr + k, wv); else wv[0] = ld_f32(wr + k);
+#pragma unroll
+        for (int t = 0; t < HLF_T; ++t) {
+            if (t >= Tn) break;
+            float xv[VL];
+            if (VEC) hl_ld16(xh + (size_t)t * x_stride + k, xv); else xv[0] = ld_f32(xh + (size_t)t * x_stride + k);
+#pragma unroll
+            for (int u = 0; u < VL; ++u) acc[t] = fmaf(xv[u], wv[u], acc[t]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < HLF_T; ++t) {
+        if (t >= Tn) break;
+        float v = acc[t];
+#pragma unroll
+        for (int o = 4; o > 0; o >>= 1) v += __shfl_xor(v, o, 8);
+        if (part == 0 && live) st_f32(out + (size_t)t * out_stride + h * out_head + n, v);
+    }
+}
+
 }  // namespace
 
 // q [T][>= H dk] is normed in place; k [T][>= Hkv dk], v [T][>= Hkv dv] go to the token's page
@@ -185,10 +238,13 @@ extern "C" int ri_head_norm_kv_write(
                              "ri_head_norm_kv_write: no keys, values or cache given, or their row strides too small");
     if (T == 0) return 0;
     RI_REQUIRE(q && positions && row_of_token, "ri_head_norm_kv_write: null pointer");
+    // a step of few tokens: a block for every four heads, so that no wave walks a chain of heads
+    const int by = T <= 256 ? min((H + Hkv + 3) / 4, 64) : 1;
+    const dim3 grid(T, by);
     if (dtype == RI_F32)
-        head_norm_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, H, Hkv, dk, dv, qw, kw, do_norm, eps, temp_coef, temp_every, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv);
+        head_norm_kv_write_kernel<float><<<grid, 256, 0, stream>>>((float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, H, Hkv, dk, dv, qw, kw, do_norm, eps, temp_coef, temp_every, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv);
     else if (dtype == RI_BF16)
-        head_norm_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, Hkv, dk, dv, qw, kw, do_norm, eps, temp_coef, temp_every, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv);
+        head_norm_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, Hkv, dk, dv, qw, kw, do_norm, eps, temp_coef, temp_every, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv);
     else
         return ri_fail("ri_head_norm_kv_write: unknown dtype %d", dtype);
     RI_LAUNCHED("ri_head_norm_kv_write");
@@ -228,6 +284,19 @@ extern "C" int ri_head_linear(const void* x, int x_stride, int x_head, const voi
     if (T == 0) return 0;
     RI_REQUIRE(x && w && out, "ri_head_linear: null pointer");
     RI_REQUIRE(H <= 65535 && (N + HL_N - 1) / HL_N <= 65535, "ri_head_linear: too many heads or outputs for the grid");
+    if (T <= HLF_T) {
+        const dim3 few((N + 31) / 32, H);
+        const int vl = dtype == RI_F32 ? 4 : 8;
+        const bool vec = K % vl == 0 && x_stride % vl == 0 && x_head % vl == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
+#define RI_HLF(TT, VV) head_linear_few_kernel<TT, VV><<<few, 256, 0, stream>>>((const TT*)x, x_stride, x_head, (const TT*)w, (TT*)out, out_stride, out_head, T, N, K)
+        if (dtype == RI_F32) { if (vec) RI_HLF(float, true); else RI_HLF(float, false); }
+        else if (dtype == RI_BF16) { if (vec) RI_HLF(bf16_t, true); else RI_HLF(bf16_t, false); }
+        else
+            return ri_fail("ri_head_linear: unknown dtype %d", dtype);
+#undef RI_HLF
+        RI_LAUNCHED("ri_head_linear");
+        return 0;
+    }
     const dim3 grid((T + HL_T - 1) / HL_T, (N + HL_N - 1) / HL_N, H);
     if (dtype == RI_F32)
         head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, x_head, (const float*)w, (float*)out, out_stride, out_head, T, N, K);

@@ -515,8 +515,10 @@ extern "C" int ri_scale_softcap(float* x, int rows, int cols, float scale, float
 // all in 32-bit.  act: null, or [rows][d] that takes the new x[r] rounded to act's dtype: the input
 // of the next sub-layer where sub-layers read the stream itself.  delta null: only that copy is made.
 // One block a row; the row's sums stay in registers between the two passes for d up to 4 * 4 * BLOCK.
+// PARTS > 0: that many partial sums, all asked for before any is added (a chain of dependent
+// loads is what a step of few rows waits for); 0: a runtime count.
 // ---------------------------------------------------------------------------
-template <typename TD, typename TW, typename TO, int BLOCK, int VEC>
+template <typename TD, typename TW, typename TO, int BLOCK, int VEC, int PARTS>
 __global__ __launch_bounds__(BLOCK) void norm_residual_kernel(
         float* __restrict__ x, const TD* __restrict__ delta, int parts, size_t part_stride, const TW* __restrict__ w,
         int one_plus, float mult, float eps, TO* __restrict__ act, int d) {
@@ -534,6 +536,18 @@ __global__ __launch_bounds__(BLOCK) void norm_residual_kernel(
     float y[CACHE][VEC];
     float ss = 0.f;
     auto sum_at = [&](int i, float* v) {
+        if (PARTS > 0) {
+            float t[PARTS > 0 ? PARTS : 1][VEC];
+#pragma unroll
+            for (int p = 0; p < PARTS; ++p) L::ld(dr + p * part_stride + i, t[p]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = t[0][e];
+#pragma unroll
+            for (int p = 1; p < PARTS; ++p)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) v[e] += t[p][e];
+            return;
+        }
         L::ld(dr + i, v);
         for (int p = 1; p < parts; ++p) {
             float t[VEC];
@@ -583,10 +597,18 @@ __global__ __launch_bounds__(BLOCK) void norm_residual_kernel(
 template <typename TD, typename TW, typename TO>
 static int launch_norm_residual(float* x, const void* delta, int parts, size_t ps, const void* w, int one_plus, float mult,
                                 float eps, void* act, int rows, int d, hipStream_t stream) {
-#define RI_NR(BLOCK, VEC) norm_residual_kernel<TD, TW, TO, BLOCK, VEC><<<rows, BLOCK, 0, stream>>>( \
+#define RI_NR_AS(BLOCK, VEC, PARTS) norm_residual_kernel<TD, TW, TO, BLOCK, VEC, PARTS><<<rows, BLOCK, 0, stream>>>( \
         x, (const TD*)delta, parts, ps, (const TW*)w, one_plus, mult, eps, (TO*)act, d)
-    if (d % 4 == 0) { if (d <= 2048) RI_NR(128, 4); else RI_NR(256, 4); }
-    else RI_NR(256, 1);
+#define RI_NR(BLOCK, VEC) do { if (!delta || parts == 1) RI_NR_AS(BLOCK, VEC, 1); else if (parts == 2) RI_NR_AS(BLOCK, VEC, 2); \
+        else if (parts == 4) RI_NR_AS(BLOCK, VEC, 4); else if (parts == 8) RI_NR_AS(BLOCK, VEC, 8); \
+        else if (parts == 16) RI_NR_AS(BLOCK, VEC, 16); else RI_NR_AS(BLOCK, VEC, 0); } while (0)
+    if (d % 4 == 0) {
+        // few rows: a row's loads are all in flight at once when every thread holds one vector of it
+        if (rows <= 256 && d >= 1024 && d <= 4096) RI_NR(1024, 4);
+        else if (d <= 2048) RI_NR(128, 4);
+        else RI_NR(256, 4);
+    } else RI_NR(256, 1);
+#undef RI_NR_AS
 #undef RI_NR
     RI_LAUNCHED("ri_norm_residual");
     return 0;

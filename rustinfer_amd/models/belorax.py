@@ -42,7 +42,7 @@ def build_belorax(cfg: BeloraxConfig) -> DecoderModel:
             mixer = LatentAttention(width, m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank, m.scale, eps,
                                     pos_enc=rotation(m.rot_dim, m.rot_base, m.rot_dims, m.rot_scaling), interleaved=True)
         elif isinstance(m, RetentionSpec):
-            mixer = Retention(width, m.heads, m.dim, m.vdim, m.decay, eps, pos_enc=rotation(m.dim, m.rot_base, m.rot_dims))
+            mixer = Retention(width, m.heads, m.dim, m.vdim, m.decay, eps, pos_enc=rotation(m.dim, m.rot_base, m.rot_dims, m.rot_scaling))
         else:
             raise TypeError(f"layer {i}: unknown mixer {m!r}")
         ffn = ffn_norm = None

@@ -167,14 +167,14 @@ def latent_attention(h, w, m, eps):
 def retention(h, w, m, eps):
     T, H, d, dv = h.shape[0], m["heads"], m["dim"], m["vdim"]
     rot = m["rot"]
-    freqs = plain_frequencies(rot["dims"], rot["base"])
+    freqs, mag = yarn_frequencies(rot["dims"], rot["base"], rot["scaling"]) if rot.get("scaling") else (plain_frequencies(rot["dims"], rot["base"]), 1.0)
     q = (h @ w["q"].T).reshape(T, H, d)
     k = (h @ w["k"].T).reshape(T, H, d)
     v = (h @ w["v"].T).reshape(T, H, dv)
     out = np.zeros((T, H, dv))
     for i in range(H):
-        qi = rotate(q[:, i], freqs, rot["dims"], False)
-        ki = rotate(k[:, i], freqs, rot["dims"], False) / math.sqrt(d)
+        qi = rotate(q[:, i], freqs, rot["dims"], False, mag)
+        ki = rotate(k[:, i], freqs, rot["dims"], False, mag) / math.sqrt(d)
         S = np.zeros((d, dv))
         for t in range(T):
             S = m["decay"][i] * S + np.outer(ki[t], v[t, i])

@@ -40,7 +40,7 @@ def test_reads_every_size_and_constant():
     assert (c.vocab_size, c.hidden_size, c.norm_eps, c.embedding_scale, c.residual_mult) == (97, 48, 3e-6, 2.5, 0.25)
     a, r, l, b = (x.mixer for x in c.layers)
     assert a == NormedAttentionSpec(6, 2, 8, 12, 0.3, 0.7, 9, None)
-    assert r == RetentionSpec(2, 16, 8, (0.9, 0.99), 777.0, 6)
+    assert r == RetentionSpec(2, 16, 8, (0.9, 0.99), 777.0, 6, None)
     assert l == LatentAttentionSpec(3, 10, 6, 14, 20, 0.2, 5000.0, 6, YarnScaling(3.0, 128, 16.0, 2.0))
     assert b == NormedAttentionSpec(2, 2, 8, 12, 0.4, 0.0, 0, 0)
     assert [x.mlp for x in c.layers] == [FeedForwardSpec("dense", 56), None, FeedForwardSpec("moe", 24, 5, 2), FeedForwardSpec("dense", 8)]
