@@ -112,7 +112,7 @@ def test_cache_books_for_these_layers():
     cm.check()
 
 
-@pytest.mark.parametrize("dims,base,sc", [(16, 1e6, dict(factor=2.0, original=1024, fast=32.0, slow=1.0)),
+@pytest.mark.parametrize("dims,base,sc", [(16, 5e5, dict(factor=3.0, original=2048, fast=16.0, slow=2.0)),
                                           (64, 1e4, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
                                           (2, 10.0, dict(factor=4.0, original=64, fast=8.0, slow=2.0)),
                                           (6, 5000.0, dict(factor=3.0, original=128, fast=16.0, slow=2.0))])

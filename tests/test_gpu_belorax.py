@@ -320,7 +320,7 @@ def test_normed_attention_alone(dtype, H, G, dk, dv, scale, coef, every, portion
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,d,r,dv,R,dims,scaling", [
-    (3, 8, 4, 12, 20, 4, None), (8, 32, 16, 32, 64, 16, dict(factor=2.0, original=64, fast=16.0, slow=1.0)),
+    (3, 8, 4, 12, 20, 4, None), (8, 32, 16, 24, 72, 16, dict(factor=2.5, original=64, fast=16.0, slow=1.0)),
     (1, 12, 6, 10, 9, 2, YARN), (5, 40, 16, 72, 136, 12, YARN), (16, 16, 8, 24, 48, 8, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
     (2, 64, 64, 130, 192, 64, YARN), (32, 4, 2, 4, 6, 2, None)])
 def test_latent_attention_alone(dtype, H, d, r, dv, R, dims, scaling, portion_kernel):
@@ -343,7 +343,7 @@ def test_latent_attention_alone(dtype, H, d, r, dv, R, dims, scaling, portion_ke
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,dk,dv,decay,dims", [(2, 16, 24, [0.9, 0.5], 16), (3, 72, 40, [0.999, 0.7, 0.2], 36), (1, 128, 64, [0.95], 2),
-                                                (4, 64, 64, [0.98, 0.99, 0.997, 0.9995], 64), (1, 256, 8, [0.9], 128), (2, 20, 130, [1.0, 0.0], 20)])
+                                                (4, 64, 48, [0.98, 0.99, 0.997, 0.9995], 32), (1, 256, 8, [0.9], 128), (2, 20, 130, [1.0, 0.0], 20)])
 def test_retention_alone(dtype, H, dk, dv, decay, dims):
     from rustinfer_amd.engine import make_runtime
     from rustinfer_amd.parts import Retention, RotaryEmbedding
@@ -361,7 +361,7 @@ def test_retention_alone(dtype, H, dk, dv, decay, dims):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("E,top,F,rows", [(4, 1, 24, 70), (16, 4, 64, 5), (70, 3, 16, 100), (6, 6, 8, 33), (3, 2, 40, 1), (130, 8, 4, 17)])
+@pytest.mark.parametrize("E,top,F,rows", [(4, 1, 24, 70), (16, 3, 56, 5), (70, 3, 16, 100), (6, 6, 8, 33), (3, 2, 40, 1), (130, 8, 4, 17)])
 def test_feed_forwards_alone(dtype, E, top, F, rows):
     from types import SimpleNamespace
     from rustinfer_amd.engine import Workspace, make_runtime
@@ -410,7 +410,7 @@ def test_yarn_tables_against_the_plain_frequencies():
     from rustinfer_amd.config import YarnScaling
     from rustinfer_amd.engine import make_runtime
     from rustinfer_amd.parts import RotaryEmbedding
-    for dims, base, sc in ((16, 1e6, dict(factor=2.0, original=1024, fast=32.0, slow=1.0)), (64, 1e4, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
+    for dims, base, sc in ((16, 5e5, dict(factor=3.0, original=2048, fast=16.0, slow=2.0)), (64, 1e4, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
                            (2, 10.0, YARN), (12, 200.0, dict(factor=2.0, original=32, fast=4.0, slow=1.0))):
         pe = RotaryEmbedding(dims, base, scaling=YarnScaling(**sc))
         pe.prepare(make_runtime("float32", DEV), 300)
