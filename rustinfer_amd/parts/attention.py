@@ -265,7 +265,8 @@ class LatentAttention(ProjectedPart, Mixer):
 
     ``pos_enc`` turns the first ``pos_enc.rot_dim`` features of a rotated part; ``interleaved``: the
     checkpoint pairs feature 2i with 2i + 1, so the rows that make the rotated parts are reordered
-    when they are loaded (even features, then odd ones), which leaves every score as it was.
+    when they are loaded (even features, then odd ones), which leaves every score as it was.  More than 32 heads run as several calls of the
+    attention kernels over the same cache.
     Tensor names: ``q, dkv, dkv.norm, uk, uv, o`` unless given."""
 
     is_mixer = True
@@ -316,9 +317,11 @@ class LatentAttention(ProjectedPart, Mixer):
     def load_own(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         n, H, R = self.names, self.num_heads, self.latent_dim
-        if not rt.ops.window_attention_supported(H, 1, R + self.rot_dim, R):
-            raise ValueError(f"latent attention with {H} heads over a latent of {R} + {self.rot_dim} features is beyond "
-                             f"the window attention kernel (32 heads, 256 features)")
+        # the attention kernels take up to 32 query heads a key/value head: more heads go in stretches of 32
+        self.heads_a_call = min(H, 32)
+        if not rt.ops.window_attention_supported(self.heads_a_call, 1, R + self.rot_dim, R):
+            raise ValueError(f"latent attention over a latent of {R} + {self.rot_dim} features is beyond the window "
+                             f"attention kernel (256 features)")
         self.norm_weight = tensors[n["norm"]].to(device=rt.device, dtype=torch.float32).contiguous()
         uk = tensors[n["uk"]].to(device=rt.device, dtype=rt.dtype)
         self.w_absorb = uk.view(H, self.head_dim, R).transpose(1, 2).contiguous()        # [H, R, head_dim]: W_uk,h^T
@@ -336,5 +339,8 @@ class LatentAttention(ProjectedPart, Mixer):
                             ctx.row_of_token, cache.k, cache.v, table, cache.page_size, write_kv=cache.write)
         ops.head_linear(q, d + r, self.w_absorb, q_lat, R + r)
         lat = ws.get("latent.sum", T, H * R, self.rt.dtype)
-        ops.window_attention(q_lat, lat, H, 1, R + r, R, cache.k, cache.v, table, cache.page_size, ctx, self.scale, 0, None, False)
+        for h0 in range(0, H, self.heads_a_call):
+            n = min(self.heads_a_call, H - h0)
+            ops.window_attention(q_lat[:, h0 * (R + r):(h0 + n) * (R + r)], lat[:, h0 * R:(h0 + n) * R], n, 1, R + r, R,
+                                 cache.k, cache.v, table, cache.page_size, ctx, self.scale, 0, None, False)
         ops.head_linear(lat, R, self.w_value, act, self.v_head_dim)

@@ -322,7 +322,7 @@ def test_normed_attention_alone(dtype, H, G, dk, dv, scale, coef, every, portion
 @pytest.mark.parametrize("H,d,r,dv,R,dims,scaling", [
     (3, 8, 4, 12, 20, 4, None), (8, 32, 16, 24, 72, 16, dict(factor=2.5, original=64, fast=16.0, slow=1.0)),
     (1, 12, 6, 10, 9, 2, YARN), (5, 40, 16, 72, 136, 12, YARN), (16, 16, 8, 24, 48, 8, dict(factor=40.0, original=4096, fast=32.0, slow=1.0)),
-    (2, 64, 64, 130, 192, 64, YARN), (32, 4, 2, 4, 6, 2, None)])
+    (2, 64, 64, 130, 192, 64, YARN), (32, 4, 2, 4, 6, 2, None), (40, 8, 4, 6, 12, 4, None)])
 def test_latent_attention_alone(dtype, H, d, r, dv, R, dims, scaling, portion_kernel):
     from rustinfer_amd.config import YarnScaling
     from rustinfer_amd.engine import make_runtime
