@@ -372,15 +372,27 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
     float m = -INFINITY, l = 0.f, acc[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) acc[c] = 0.f;
-    for (int s = 0; s < n && s < slots; ++s) {
-        const size_t at = ((size_t)t * H + h) * slots + s;
-        float acc_b[NC];
+    // eight blocks' partial results are asked for at once, then merged one after the other in the
+    // order of the blocks: the loads of a block do not wait for the merge of the one before
+    constexpr int AHEAD = 8;
+    const int count = min(n, slots);
+    for (int s0 = 0; s0 < count; s0 += AHEAD) {
+        float acc_b[AHEAD][NC], m_b[AHEAD], l_b[AHEAD];
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            const int d = lane + 64 * c;
-            acc_b[c] = d < dv ? part_o[at * dv + d] : 0.f;
+        for (int i = 0; i < AHEAD; ++i) {
+            const bool on = s0 + i < count;
+            const size_t at = ((size_t)t * H + h) * slots + (on ? s0 + i : s0);
+            m_b[i] = on ? part_ml[at * 2] : -INFINITY;
+            l_b[i] = on ? part_ml[at * 2 + 1] : 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const int d = lane + 64 * c;
+                acc_b[i][c] = (on && d < dv) ? part_o[at * dv + d] : 0.f;
+            }
         }
-        aw_merge<NC>(m, l, acc, part_ml[at * 2], part_ml[at * 2 + 1], acc_b);
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i)
+            if (s0 + i < count) aw_merge<NC>(m, l, acc, m_b[i], l_b[i], acc_b[i]);
     }
     T* o = out + (size_t)t * out_stride + h * dv;
 #pragma unroll
