@@ -7,6 +7,9 @@
 //                       the experts' activations side by side, each scaled by its token's weight, so
 //                       that ONE product with the experts' down matrices side by side is the weighted
 //                       sum of the chosen experts' outputs (an expert that was not chosen adds zeros).
+//   moe_swiglu_routed   the two in one launch: every block makes its token's weights from the logits
+//                       itself (what the engine runs; the two above are its halves, kept for callers
+//                       that want the weights).
 #include "common.h"
 #include <math.h>
 
@@ -14,11 +17,8 @@ namespace {
 
 constexpr int MOE_EPL = 8;       // experts a lane: up to 512 experts
 
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int l_stride, float* __restrict__ weights,
-                                                       int T, int E, int top, int renorm) {
-    const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= T) return;
-    const float* z = logits + (size_t)t * l_stride;
+// One wave: the weights of a token's experts from its logits z [E] into wr [E] (global or LDS).
+__device__ __forceinline__ void route_token(const float* __restrict__ z, float* wr, int E, int top, int renorm, int lane) {
     float s[MOE_EPL];
     float m = -INFINITY;
 #pragma unroll
@@ -56,12 +56,41 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         kept += best * inv;
     }
     const float f = renorm ? inv / kept : inv;
-    float* wr = weights + (size_t)t * E;
 #pragma unroll
     for (int j = 0; j < MOE_EPL; ++j) {
         const int e = lane + 64 * j;
         if (e < E) wr[e] = (chosen >> j & 1u) ? s[j] * f : 0.f;
     }
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int l_stride, float* __restrict__ weights,
+                                                       int T, int E, int top, int renorm) {
+    const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    route_token(logits + (size_t)t * l_stride, weights + (size_t)t * E, E, top, renorm, lane);
+}
+
+// moe_swiglu_weighted with the routing done on the way: the block's first wave makes the token's weights
+// from its logits into LDS (every block of a token the same ones), then all threads use them.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_swiglu_routed_kernel(const T* __restrict__ gu, int gu_stride, const float* __restrict__ logits,
+                                                               int l_stride, T* __restrict__ act, int act_stride, int E, int F,
+                                                               int top, int renorm) {
+    __shared__ float wts[64 * MOE_EPL];
+    const int t = blockIdx.y;
+    if (threadIdx.x < 64) route_token(logits + (size_t)t * l_stride, wts, E, top, renorm, threadIdx.x);
+    __syncthreads();
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= E * F) return;
+    const int e = idx / F, i = idx - e * F;
+    const float wgt = wts[e];
+    float y = 0.f;
+    if (wgt != 0.f) {
+        const T* row = gu + (size_t)t * gu_stride + (size_t)e * 2 * F;
+        const float g = ld_f32(row + i), u = ld_f32(row + F + i);
+        y = wgt * (g / (1.f + expf(-g))) * u;
+    }
+    st_f32(act + (size_t)t * act_stride + idx, y);
 }
 
 template <typename T>
@@ -104,5 +133,21 @@ extern "C" int ri_moe_swiglu_weighted(const void* gu, int gu_stride, const float
     else if (dtype == RI_BF16) moe_swiglu_weighted_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gu, gu_stride, weights, (bf16_t*)act, act_stride, E, F);
     else return ri_fail("ri_moe_swiglu_weighted: unknown dtype %d", dtype);
     RI_LAUNCHED("ri_moe_swiglu_weighted");
+    return 0;
+}
+
+// The two in one launch: act from gate_up and the router's 32-bit logits [T][>= E].
+extern "C" int ri_moe_swiglu_routed(const void* gu, int gu_stride, const float* logits, int l_stride, void* act, int act_stride,
+                                    int dtype, int T, int E, int F, int top, int renorm, hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && E > 0 && F > 0 && gu_stride >= 2 * E * F && act_stride >= E * F && l_stride >= E, "ri_moe_swiglu_routed: bad sizes");
+    RI_REQUIRE(top > 0 && top <= E && E <= 64 * MOE_EPL, "ri_moe_swiglu_routed: top %d of %d experts (up to %d)", top, E, 64 * MOE_EPL);
+    if (T == 0) return 0;
+    RI_REQUIRE(gu && logits && act, "ri_moe_swiglu_routed: null pointer");
+    RI_REQUIRE(T <= 65535, "ri_moe_swiglu_routed: too many rows for the grid");
+    const dim3 grid((E * F + 255) / 256, T);
+    if (dtype == RI_F32) moe_swiglu_routed_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, gu_stride, logits, l_stride, (float*)act, act_stride, E, F, top, renorm);
+    else if (dtype == RI_BF16) moe_swiglu_routed_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gu, gu_stride, logits, l_stride, (bf16_t*)act, act_stride, E, F, top, renorm);
+    else return ri_fail("ri_moe_swiglu_routed: unknown dtype %d", dtype);
+    RI_LAUNCHED("ri_moe_swiglu_routed");
     return 0;
 }

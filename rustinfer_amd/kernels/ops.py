@@ -1183,3 +1183,19 @@ def moe_swiglu_weighted(gate_up: torch.Tensor, weights: torch.Tensor, act: torch
         raise KernelError("moe_swiglu_weighted: gate_up [T, 2 E F], 32-bit weights [T, E] and act [T, E F] expected")
     _check(_lib().ri_moe_swiglu_weighted(_ptr(gate_up), gate_up.stride(0), _ptr(weights), _ptr(act), act.stride(0),
                                          _dt(act), T, E, F, _stream()))
+
+
+def moe_swiglu_routed(gate_up: torch.Tensor, logits: torch.Tensor, act: torch.Tensor, E: int, F: int, top: int,
+                      renormalize: bool = False) -> None:
+    """``moe_route`` and ``moe_swiglu_weighted`` in one launch: the weights are made from the 32-bit
+    ``logits [T, E]`` on the way and never stored."""
+    _dev(gate_up, logits, act)
+    _rows2d(gate_up, "gate_up")
+    _rows2d(act, "act")
+    _rows2d(logits, "logits")
+    T = gate_up.shape[0]
+    if gate_up.shape[1] != 2 * E * F or tuple(act.shape) != (T, E * F) or act.dtype != gate_up.dtype \
+            or logits.dtype != torch.float32 or tuple(logits.shape) != (T, E):
+        raise KernelError("moe_swiglu_routed: gate_up [T, 2 E F], 32-bit logits [T, E] and act [T, E F] expected")
+    _check(_lib().ri_moe_swiglu_routed(_ptr(gate_up), gate_up.stride(0), _ptr(logits), logits.stride(0), _ptr(act),
+                                       act.stride(0), _dt(act), T, E, F, int(top), int(bool(renormalize)), _stream()))

@@ -109,11 +109,16 @@ class MoEFeedForward(FeedForward):
 
     The experts' gate and up matrices are stacked into one product for all of them, every expert's
     activation is multiplied by its token's weight (0 where it was not chosen), and the experts' down
-    matrices side by side make the weighted sum in ONE product: three launches whatever the number of
-    experts, nothing that depends on which experts a token chose (so a step can be captured), and
+    matrices side by side make the weighted sum in ONE product: the router's product and three more
+    launches whatever the number of experts, nothing that depends on which experts a token chose (so a step can be captured), and
     the same arithmetic for a token whatever else is in the step.  Every token pays for all experts;
     with few tokens in a step the experts' weights are read once either way.
     Tensor names: ``router``, ``e<i>.gate``, ``e<i>.up``, ``e<i>.down``."""
+
+    # up to this many tokens in a step every block of the activation kernel makes its token's weights
+    # itself (a launch less: 4.6 us of a step of 8 tokens); with more, the weights are made once a token
+    # by a kernel of their own (a prompt of 2,048 tokens: 81 against 250 us a layer)
+    ROUTE_ON_THE_WAY_ROWS = 64
 
     def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, renormalize: bool = False):
         if not (0 < top <= experts):
@@ -143,10 +148,13 @@ class MoEFeedForward(FeedForward):
         T, E, F = normed.shape[0], self.experts, self.expert_size
         logits = ws.get("moe.logits", T, E, torch.float32)
         self.router.forward(normed, logits)
-        weights = ws.get("moe.weights", T, E, torch.float32)
-        ops.moe_route(logits, weights, self.top, self.renormalize)
         gate_up = ws.get("moe.gate_up", T, 2 * E * F, self.rt.dtype)
         self.gate_up.forward(normed, gate_up)
         act = ws.get("moe.act", T, E * F, self.rt.dtype)
-        ops.moe_swiglu_weighted(gate_up, weights, act, E, F)
+        if T <= self.ROUTE_ON_THE_WAY_ROWS:
+            ops.moe_swiglu_routed(gate_up, logits, act, E, F, self.top, self.renormalize)
+        else:
+            weights = ws.get("moe.weights", T, E, torch.float32)
+            ops.moe_route(logits, weights, self.top, self.renormalize)
+            ops.moe_swiglu_weighted(gate_up, weights, act, E, F)
         return ops.linear_delta(act, self.down.weight, ws, "moe.out", self.down.weight_tiled, out_dtype=torch.float32)

@@ -387,6 +387,33 @@ def test_feed_forwards_alone(dtype, E, top, F, rows):
     assert rel(out.cpu().numpy(), P.gated_ff(x.double().numpy(), w)) < PART_TOL[dtype]
 
 
+@pytest.mark.parametrize("E,top,F,renorm", [(8, 2, 32, False), (70, 5, 3, True), (300, 300, 2, False), (5, 1, 7, True)])
+def test_routing_kernels(E, top, F, renorm):
+    """The weights of ``moe_route`` against a plain softmax and sort, and the launch that routes on the
+    way against the two kernels it stands for."""
+    from rustinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(E)
+    T = 37
+    logits = (torch.randn(T, E, generator=g) * 3.0).to(DEV)
+    gate_up = torch.randn(T, 2 * E * F, generator=g).to(DEV)
+    weights = torch.empty(T, E, device=DEV)
+    ops.moe_route(logits, weights, top, renorm)
+    z = logits.double().cpu().numpy()
+    prob = P.softmax_rows(z)
+    want = np.zeros_like(prob)
+    for t in range(T):
+        keep = np.argsort(-prob[t], kind="stable")[:top]
+        want[t, keep] = prob[t, keep] / (prob[t, keep].sum() if renorm else 1.0)
+    assert np.abs(weights.double().cpu().numpy() - want).max() < 1e-6
+    two, one = torch.empty(T, E * F, device=DEV), torch.empty(T, E * F, device=DEV)
+    ops.moe_swiglu_weighted(gate_up, weights, two, E, F)
+    ops.moe_swiglu_routed(gate_up, logits, one, E, F, top, renorm)
+    assert torch.equal(one, two)
+    gu = gate_up.double().cpu().numpy().reshape(T, E, 2, F)
+    ref = (want[:, :, None] * P.silu(gu[:, :, 0]) * gu[:, :, 1]).reshape(T, E * F)
+    assert rel(one.double().cpu().numpy(), ref) < 2e-6
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("width,parts", [(64, 1), (100, 3), (4096 + 8, 2), (33, 1)])
 def test_the_norm_on_a_sublayers_output(dtype, width, parts):
